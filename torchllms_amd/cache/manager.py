@@ -46,6 +46,11 @@ class CacheGroupSpec:
     window: int = 0  # 0: all keys stay; w > 0: only the last w positions are read
     page_size: int = 0  # tokens per page; 0: the manager's default
     dtype: Optional[str] = None  # "float32" / "bfloat16"; None: the manager's default
+    v_head_dim: int = 0  # head size of the values; 0: that of the keys
+
+    @property
+    def value_dim(self) -> int:
+        return self.v_head_dim or self.head_dim
 
 
 @dataclass(frozen=True)
@@ -68,16 +73,18 @@ def group_layers(needs: Sequence[Tuple[Hashable, object]]) -> Tuple[List[CacheGr
         if need is None:
             continue
         if hasattr(need, "num_kv_heads"):
+            v_dim = int(getattr(need, "v_head_dim", None) or 0)
             form = (need.num_kv_heads, need.head_dim, need.window, int(getattr(need, "page_size", None) or 0),
-                    getattr(need, "dtype", None))
+                    getattr(need, "dtype", None), 0 if v_dim == need.head_dim else v_dim)
             kv.setdefault(form, []).append(run_id)
         elif hasattr(need, "shape"):
             st.setdefault((tuple(need.shape), need.dtype), []).append(run_id)
         else:
             raise TypeError(f"cache entry {run_id}: unknown cache need {need!r}")
     groups = [
-        CacheGroupSpec(name=f"kv{i}", run_ids=tuple(runs), num_kv_heads=h, head_dim=d, window=w, page_size=p, dtype=t)
-        for i, ((h, d, w, p, t), runs) in enumerate(kv.items())
+        CacheGroupSpec(name=f"kv{i}", run_ids=tuple(runs), num_kv_heads=h, head_dim=d, window=w, page_size=p, dtype=t,
+                       v_head_dim=vd)
+        for i, ((h, d, w, p, t, vd), runs) in enumerate(kv.items())
     ]
     states = [
         StateSlotSpec(name=f"state{i}", run_ids=tuple(runs), shape=shape, dtype=dtype)
@@ -147,7 +154,7 @@ class KVLayerView:
 
     group: int
     k_pages: torch.Tensor  # [num_pages, Hkv, page_size, dh]
-    v_pages: torch.Tensor
+    v_pages: torch.Tensor  # [num_pages, Hkv, page_size, dh of the values]
     page_size: int
     writes: bool = True  # False when this run borrows another run's cache
 
@@ -211,9 +218,9 @@ class CacheManager:
         self.state_tensors: List[Optional[torch.Tensor]] = []
         if device is not None:
             for gi, (g, pool) in enumerate(zip(self.groups, self.pools)):
-                shape = (len(g.run_ids), pool.num_pages, g.num_kv_heads, self.page_sizes[gi], g.head_dim)
-                self.k_pages.append(torch.zeros(shape, dtype=self.dtypes[gi], device=device))
-                self.v_pages.append(torch.zeros(shape, dtype=self.dtypes[gi], device=device))
+                shape = (len(g.run_ids), pool.num_pages, g.num_kv_heads, self.page_sizes[gi])
+                self.k_pages.append(torch.zeros(shape + (g.head_dim,), dtype=self.dtypes[gi], device=device))
+                self.v_pages.append(torch.zeros(shape + (g.value_dim,), dtype=self.dtypes[gi], device=device))
             for s in self.states:
                 shape = (len(s.run_ids), max_seqs, *s.shape)
                 self.state_tensors.append(torch.zeros(shape, dtype=getattr(torch, s.dtype), device=device))
@@ -226,7 +233,7 @@ class CacheManager:
         total = 0
         for g in groups:
             elt = torch.empty(0, dtype=getattr(torch, g.dtype) if g.dtype else dtype).element_size()
-            total += 2 * len(g.run_ids) * g.num_kv_heads * g.head_dim * elt
+            total += len(g.run_ids) * g.num_kv_heads * (g.head_dim + g.value_dim) * elt
         return total
 
     @staticmethod
@@ -452,7 +459,7 @@ class CacheManager:
         page_size = self.page_sizes[gi]
         n = e.num_tokens
         k = torch.zeros((n, g.num_kv_heads, g.head_dim), dtype=self.dtypes[gi], device=self.device)
-        v = torch.zeros_like(k)
+        v = torch.zeros((n, g.num_kv_heads, g.value_dim), dtype=self.dtypes[gi], device=self.device)
         for b, page in enumerate(e.block_tables[gi]):
             lo = b * page_size
             hi = min(lo + page_size, n)

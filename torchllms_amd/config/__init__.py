@@ -8,6 +8,7 @@ from .registry import (
     load_config,
     register_architecture,
 )
+from .taluvik import TaluvikConfig, TaluvikLayer, taluvik_model_spec
 from .spec import LayerRun, LayerSpec, ModelSpec, PartSpec, standard_layer
 
 __all__ = [
@@ -20,6 +21,9 @@ __all__ = [
     "ModelSpec",
     "PartSpec",
     "RopeScaling",
+    "TaluvikConfig",
+    "TaluvikLayer",
+    "taluvik_model_spec",
     "architecture_name",
     "architecture_of",
     "get_architecture",

@@ -16,6 +16,7 @@ from typing import Any, Callable, Dict, List, Optional, Sequence
 
 from .llama import ConfigError, LlamaConfig, llama_model_spec
 from .spec import ModelSpec
+from .taluvik import ARCHITECTURE as TALUVIK, TaluvikConfig, taluvik_model_spec
 
 
 @dataclass(frozen=True)
@@ -53,7 +54,7 @@ class ArchSpec:
             import dataclasses
 
             d = dataclasses.asdict(config)
-        if not d.get("architectures"):
+        if not d.get("architectures") and not d.get("architecture"):
             d["architectures"] = [self.name]
         return d
 
@@ -95,10 +96,14 @@ def architecture_of(config) -> ArchSpec:
 
 
 def architecture_name(config_dict: Dict[str, Any]) -> str:
+    """The architecture a config.json names: the first of "architectures", or the string "architecture"."""
     archs = config_dict.get("architectures")
-    if not archs:
-        raise ConfigError('config.json has no "architectures" entry')
-    return archs[0]
+    if archs:
+        return archs[0]
+    one = config_dict.get("architecture")
+    if isinstance(one, str) and one:
+        return one
+    raise ConfigError('config.json names no architecture ("architectures" or "architecture")')
 
 
 def load_config(folder) -> tuple:
@@ -133,5 +138,28 @@ register_architecture(
         weight_rules=_llama_rules,
         stop_token_ids=_llama_stop_ids,
         config_type=LlamaConfig,
+    )
+)
+
+
+def _taluvik_rules(cfg: TaluvikConfig):
+    from ..weights.names import taluvik_name_rules
+
+    return taluvik_name_rules(cfg)
+
+
+def _taluvik_stop_ids(cfg: TaluvikConfig):
+    eos = cfg.eos_token_id
+    return [] if eos is None else (list(eos) if isinstance(eos, (list, tuple)) else [eos])
+
+
+register_architecture(
+    ArchSpec(
+        name=TALUVIK,
+        config_from_dict=TaluvikConfig.from_dict,
+        model_spec=taluvik_model_spec,
+        weight_rules=_taluvik_rules,
+        stop_token_ids=_taluvik_stop_ids,
+        config_type=TaluvikConfig,
     )
 )

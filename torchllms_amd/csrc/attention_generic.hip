@@ -3,7 +3,10 @@
 // (token, query head).  Keys are visited in ascending position in blocks of 64 aligned to
 // absolute position, so a result depends only on the query's position and the cache contents,
 // never on how the step was batched.  This is the kernel of the 32-bit path and the fallback of
-// the bfloat16 path for sizes the MFMA kernels refuse.
+// the bfloat16 path for sizes the MFMA kernels refuse.  Beyond the plain form it takes: values of
+// another head size than the keys (v_dim), a cap on the scores (s <- cap * tanh(s / cap)), chunks
+// (a query sees only keys of its own chunk of `chunk` positions, counted from position 0) and a sink
+// per query head (one more term exp(sink) in the softmax's denominator, without a value).
 #include <limits.h>
 
 #include "common.h"
@@ -47,11 +50,26 @@ struct Query {
   const T* k_pages;
   const T* v_pages;
   const int32_t* bt;        // the request's block table
-  int n_kv_heads, g, head_dim, page_size;
-  size_t head_elems;
+  int n_kv_heads, g, head_dim, v_dim, page_size;
   int lo, p;                // the keys it sees: positions lo .. p
-  float scale;
+  float scale, softcap;
 };
+
+// The first position a query at position p sees: behind a window of `window` keys (0: none) and inside
+// its own chunk of `chunk` positions (0: none).
+__device__ __forceinline__ int first_key(int p, int window, int chunk) {
+  int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (chunk > 0) lo = max(lo, p - p % chunk);
+  return lo;
+}
+
+// The score as the softmax takes it.
+__device__ __forceinline__ float capped(float s, float softcap) { return softcap > 0.f ? softcap * tanhf(s / softcap) : s; }
+
+// The sum of probabilities with the sink's term, relative to the running maximum m.
+__device__ __forceinline__ float with_sink(float l, float m, const float* sinks, int h) {
+  return sinks ? l + expf(sinks[h] - m) : l;
+}
 
 // One block of 64 keys (positions j0 .. j0 + 63, j0 a multiple of 64), by one wave, all in 32-bit:
 //   s_j = scale * (q . k_j), products chained from channel 0 up;  m = max_j s_j;  p_j = exp(s_j - m);
@@ -67,11 +85,11 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
   const int j = j0 + lane;
   const bool valid = j >= a.lo && j <= a.p;
   float s = -INFINITY;
-  long long row_at = 0;  // element offset of this lane's key (and value) row in the pages
+  long long row_at = 0;  // index of this lane's key (and value) row in the pages
   if (valid) {
     const int page = a.bt[j / a.page_size];
-    row_at = (long long)(((size_t)page * a.n_kv_heads + a.g) * a.head_elems + (size_t)(j % a.page_size) * a.head_dim);
-    const T* kr = a.k_pages + row_at;
+    row_at = (long long)(((size_t)page * a.n_kv_heads + a.g) * a.page_size + (size_t)(j % a.page_size));
+    const T* kr = a.k_pages + row_at * a.head_dim;
     float dot = 0.f;
     if (VEC) {
       // eight pieces of the row are asked for before the first is multiplied (a piece past the row's end is
@@ -96,7 +114,7 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
     } else {
       for (int d = 0; d < a.head_dim; ++d) dot = fmaf(a.qs[d], to_f32(kr[d]), dot);
     }
-    s = dot * a.scale;
+    s = capped(dot * a.scale, a.softcap);
   }
   m_b = wave_max(s);
   const float pj = valid ? expf(s - m_b) : 0.f;
@@ -114,12 +132,12 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int src = jj + u <= jj_hi ? jj + u : jj_hi;  // rows past the end: fetched again, never added
-      const T* vr = a.v_pages + __shfl(row_at, src, kWave);
+      const T* vr = a.v_pages + __shfl(row_at, src, kWave) * a.v_dim;
       pw[u] = __shfl(pj, src, kWave);
 #pragma unroll
       for (int c = 0; c < kChanPerLane; ++c) {
         const int d = lane + c * kWave;
-        if (c * kWave < a.head_dim) vv[u][c] = vr[d < a.head_dim ? d : 0];
+        if (c * kWave < a.v_dim) vv[u][c] = vr[d < a.v_dim ? d : 0];
       }
     }
 #pragma unroll
@@ -128,7 +146,7 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
 #pragma unroll
         for (int c = 0; c < kChanPerLane; ++c) {
           const int d = lane + c * kWave;
-          if (c * kWave < a.head_dim) o_b[c] = fmaf(pw[u], d < a.head_dim ? to_f32(vv[u][c]) : 0.f, o_b[c]);
+          if (c * kWave < a.v_dim) o_b[c] = fmaf(pw[u], d < a.v_dim ? to_f32(vv[u][c]) : 0.f, o_b[c]);
         }
       }
   }
@@ -152,15 +170,16 @@ template <typename T>
 __device__ __forceinline__ Query<T> make_query(const float* qs, const T* k_pages, const T* v_pages,
                                                const int32_t* token_seq, const int32_t* positions,
                                                const int32_t* block_table, int bt_stride, int t, int h, int n_q_heads,
-                                               int n_kv_heads, int head_dim, int page_size, int window, float scale) {
+                                               int n_kv_heads, int head_dim, int page_size, int window, float scale,
+                                               float softcap, int chunk, int v_dim) {
   Query<T> a;
   a.qs = qs; a.k_pages = k_pages; a.v_pages = v_pages;
   a.bt = block_table + (size_t)token_seq[t] * bt_stride;
-  a.n_kv_heads = n_kv_heads; a.g = h / (n_q_heads / n_kv_heads); a.head_dim = head_dim; a.page_size = page_size;
-  a.head_elems = (size_t)page_size * head_dim;
+  a.n_kv_heads = n_kv_heads; a.g = h / (n_q_heads / n_kv_heads); a.head_dim = head_dim; a.v_dim = v_dim;
+  a.page_size = page_size;
   a.p = positions[t];
-  a.lo = (window > 0 && a.p - window + 1 > 0) ? a.p - window + 1 : 0;
-  a.scale = scale;
+  a.lo = first_key(a.p, window, chunk);
+  a.scale = scale; a.softcap = softcap;
   return a;
 }
 
@@ -172,7 +191,8 @@ attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
                          const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                          const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ block_table, int bt_stride, int n_q_heads,
-                         int n_kv_heads, int head_dim, int page_size, int window, float scale) {
+                         int n_kv_heads, int head_dim, int page_size, int window, float scale, float softcap,
+                         int chunk, const float* __restrict__ sinks, int v_dim) {
   __shared__ float q_lds[kWavesPerBlock][kMaxHeadDim];
   const int t = blockIdx.x;
   const int wave = threadIdx.x / kWave;
@@ -184,7 +204,7 @@ attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave][d] = to_f32(qv[d]);
   __syncthreads();
   const Query<T> a = make_query<T>(q_lds[wave], k_pages, v_pages, token_seq, positions, block_table, bt_stride, t, h,
-                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale);
+                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim);
   float acc[kChanPerLane];
 #pragma unroll
   for (int c = 0; c < kChanPerLane; ++c) acc[c] = 0.f;
@@ -195,12 +215,12 @@ attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
     merge_block(m, l, acc, m_b, l_b, o_b);
   }
   if (active) {
-    T* o = out + (size_t)t * out_stride + (size_t)h * head_dim;
-    const float inv_l = 1.0f / l;
+    T* o = out + (size_t)t * out_stride + (size_t)h * v_dim;
+    const float inv_l = 1.0f / with_sink(l, m, sinks, h);
 #pragma unroll
     for (int c = 0; c < kChanPerLane; ++c) {
       const int d = lane + c * kWave;
-      if (d < head_dim) o[d] = from_f32<T>(acc[c] * inv_l);
+      if (d < v_dim) o[d] = from_f32<T>(acc[c] * inv_l);
     }
   }
 }
@@ -217,7 +237,8 @@ constexpr int kTilePad = 4;  // floats between LDS rows beyond head_dim: rows st
 
 template <bool VEC, int CH>
 __device__ __forceinline__ void block_partial_lds(const float* qs, const float* k_t, const float* v_t, int pitch,
-                                                  int head_dim, int lo, int p, float scale, int j0, int lane,
+                                                  int pitch_v, int head_dim, int v_dim, int lo, int p, float scale,
+                                                  float softcap, int j0, int lane,
                                                   float& m_b, float& l_b, float (&o_b)[kChanPerLane]) {
 #pragma clang fp contract(off)
   const int j = j0 + lane;
@@ -236,7 +257,7 @@ __device__ __forceinline__ void block_partial_lds(const float* qs, const float* 
     } else {
       for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], kr[d], dot);
     }
-    s = dot * scale;
+    s = capped(dot * scale, softcap);
   }
   m_b = wave_max(s);
   const float pj = valid ? expf(s - m_b) : 0.f;
@@ -250,7 +271,7 @@ __device__ __forceinline__ void block_partial_lds(const float* qs, const float* 
   // they add zeros).
   auto value = [&](int jj, int c) {
     const int d = lane + c * kWave;
-    return (c + 1 < CH || d < head_dim) ? v_t[jj * pitch + d] : 0.f;
+    return (c + 1 < CH || d < v_dim) ? v_t[jj * pitch_v + d] : 0.f;
   };
   constexpr int U = 4;  // value rows asked for together; they are still added one after the other
   int jj = jj_lo;
@@ -280,12 +301,13 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
                       const T* __restrict__ k_pages, const T* __restrict__ v_pages,
                       const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                       const int32_t* __restrict__ block_table, int bt_stride, int n_tokens, int n_q_heads,
-                      int n_kv_heads, int head_dim, int page_size, int window, float scale, int heads_per_block) {
+                      int n_kv_heads, int head_dim, int page_size, int window, float scale, int heads_per_block,
+                      float softcap, int chunk, const float* __restrict__ sinks, int v_dim) {
   extern __shared__ __attribute__((aligned(16))) float tile_lds[];
-  const int pitch = head_dim + kTilePad;
+  const int pitch = head_dim + kTilePad, pitch_v = v_dim + kTilePad;
   float* q_lds = tile_lds;                          // [kTileWaves][head_dim]
   float* k_t = tile_lds + kTileWaves * head_dim;    // [64][pitch]
-  float* v_t = k_t + kWave * pitch;                 // [64][pitch]
+  float* v_t = k_t + kWave * pitch;                 // [64][pitch_v]
   const int HB = heads_per_block;
   const int QT = kTileWaves / HB;
   const int wave = threadIdx.x / kWave;
@@ -299,7 +321,8 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
   const T* qv = q + (size_t)t * q_stride + (size_t)h * head_dim;
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave * head_dim + d] = to_f32(qv[d]);
   const Query<T> a = make_query<T>(q_lds + wave * head_dim, k_pages, v_pages, token_seq, positions, block_table,
-                                   bt_stride, t, h, n_q_heads, n_kv_heads, head_dim, page_size, window, scale);
+                                   bt_stride, t, h, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap,
+                                   chunk, v_dim);
   // what the whole block sees: the same for every thread, from the tokens' own entries
   const int last = min(t0 + QT, n_tokens) - 1;
   const int seq0 = token_seq[t0];
@@ -308,7 +331,7 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
   for (int i = t0; i <= last; ++i) {
     together = together && token_seq[i] == seq0;
     const int pi = positions[i];
-    const int li = (window > 0 && pi - window + 1 > 0) ? pi - window + 1 : 0;
+    const int li = first_key(pi, window, chunk);
     blk_lo = min(blk_lo, li - li % kWave);
     key_lo = min(key_lo, li);
     blk_hi = max(blk_hi, pi);
@@ -329,43 +352,46 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
   } else {
     const int g = (blockIdx.y * HB) / (n_q_heads / n_kv_heads);  // the kv head of all the block's heads
     const int32_t* bt = block_table + (size_t)seq0 * bt_stride;
-    const size_t head_elems = (size_t)page_size * head_dim;
-    const int per_row = VEC ? head_dim / 4 : head_dim;  // pieces of a row: four elements, or one
+    // pieces of a key row and of a value row: four elements, or one
+    const int per_k = VEC ? head_dim / 4 : head_dim, per_v = VEC ? v_dim / 4 : v_dim;
+    const int per_row = per_k + per_v;
     for (int j0 = blk_lo; j0 <= blk_hi; j0 += kWave) {
       if (j0 > blk_lo) __syncthreads();  // everybody has finished with the tiles of the block before
       for (int idx = threadIdx.x; idx < kWave * per_row; idx += kTileWaves * kWave) {
-        const int r = idx / per_row, piece = idx % per_row;
+        const int r = idx / per_row, piece_kv = idx % per_row;
         const int j = j0 + r;
         if (j < key_lo || j > blk_hi) continue;  // nobody in the block sees this key
         const int page = bt[j / page_size];
         if (page < 0) continue;  // a page that a window gave back: no token of the step sees its keys
-        const size_t row_at = ((size_t)page * n_kv_heads + g) * head_elems + (size_t)(j % page_size) * head_dim;
+        const size_t row_at = ((size_t)page * n_kv_heads + g) * page_size + (size_t)(j % page_size);
+        const bool is_k = piece_kv < per_k;
+        const int piece = is_k ? piece_kv : piece_kv - per_k;
+        const T* src = is_k ? k_pages + row_at * head_dim : v_pages + row_at * v_dim;
+        float* dst = is_k ? k_t + r * pitch : v_t + r * pitch_v;
         if (VEC) {
-          float kv[4], vv[4];
-          load4(k_pages + row_at + 4 * piece, kv);
-          load4(v_pages + row_at + 4 * piece, vv);
-          *reinterpret_cast<float4*>(k_t + r * pitch + 4 * piece) = float4{kv[0], kv[1], kv[2], kv[3]};
-          *reinterpret_cast<float4*>(v_t + r * pitch + 4 * piece) = float4{vv[0], vv[1], vv[2], vv[3]};
+          float e[4];
+          load4(src + 4 * piece, e);
+          *reinterpret_cast<float4*>(dst + 4 * piece) = float4{e[0], e[1], e[2], e[3]};
         } else {
-          k_t[r * pitch + piece] = to_f32(k_pages[row_at + piece]);
-          v_t[r * pitch + piece] = to_f32(v_pages[row_at + piece]);
+          dst[piece] = to_f32(src[piece]);
         }
       }
       __syncthreads();
       if (j0 >= lo_u - lo_u % kWave && j0 <= p_u) {  // (uniform per wave)
         float m_b, l_b, o_b[kChanPerLane];
-        block_partial_lds<VEC, CH>(a.qs, k_t, v_t, pitch, head_dim, lo_u, p_u, scale, j0, lane, m_b, l_b, o_b);
+        block_partial_lds<VEC, CH>(a.qs, k_t, v_t, pitch, pitch_v, head_dim, v_dim, lo_u, p_u, scale, softcap, j0, lane,
+                                   m_b, l_b, o_b);
         merge_block(m, l, acc, m_b, l_b, o_b);
       }
     }
   }
   if (active) {
-    T* o = out + (size_t)t * out_stride + (size_t)h * head_dim;
-    const float inv_l = 1.0f / l;
+    T* o = out + (size_t)t * out_stride + (size_t)h * v_dim;
+    const float inv_l = 1.0f / with_sink(l, m, sinks, h);
 #pragma unroll
     for (int c = 0; c < kChanPerLane; ++c) {
       const int d = lane + c * kWave;
-      if (d < head_dim) o[d] = from_f32<T>(acc[c] * inv_l);
+      if (d < v_dim) o[d] = from_f32<T>(acc[c] * inv_l);
     }
   }
 }
@@ -382,7 +408,7 @@ attention_blocks_kernel(const T* __restrict__ q, int q_stride, const T* __restri
                         const T* __restrict__ v_pages, const int32_t* __restrict__ token_seq,
                         const int32_t* __restrict__ positions, const int32_t* __restrict__ block_table, int bt_stride,
                         int n_q_heads, int n_kv_heads, int head_dim, int page_size, int window, float scale,
-                        float* __restrict__ partials, int max_blocks) {
+                        float* __restrict__ partials, int max_blocks, float softcap, int chunk, int v_dim) {
   __shared__ float q_lds[kWavesPerBlock][kMaxHeadDim];
   const int t = blockIdx.x;
   const int r = blockIdx.z;
@@ -395,34 +421,35 @@ attention_blocks_kernel(const T* __restrict__ q, int q_stride, const T* __restri
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave][d] = to_f32(qv[d]);
   __syncthreads();
   const Query<T> a = make_query<T>(q_lds[wave], k_pages, v_pages, token_seq, positions, block_table, bt_stride, t, h,
-                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale);
+                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim);
   const int j0 = a.lo - a.lo % kWave + r * kWave;
   if (j0 > a.p || !active) return;  // (uniform per wave)
   float m_b, l_b, o_b[kChanPerLane];
   block_partial<T, VEC>(a, j0, lane, m_b, l_b, o_b);
-  float* dst = partials + (((size_t)t * n_q_heads + h) * max_blocks + r) * (head_dim + kPartialExtra);
+  float* dst = partials + (((size_t)t * n_q_heads + h) * max_blocks + r) * (v_dim + kPartialExtra);
 #pragma unroll
   for (int c = 0; c < kChanPerLane; ++c) {
     const int d = lane + c * kWave;
-    if (d < head_dim) dst[d] = o_b[c];
+    if (d < v_dim) dst[d] = o_b[c];
   }
   if (lane == 0) {
-    dst[head_dim] = m_b;
-    dst[head_dim + 1] = l_b;
+    dst[v_dim] = m_b;
+    dst[v_dim + 1] = l_b;
   }
 }
 
 template <typename T>
 __global__ void __launch_bounds__(kWavesPerBlock* kWave)
 attention_join_kernel(T* __restrict__ out, int out_stride, const int32_t* __restrict__ positions, int n_q_heads,
-                      int head_dim, int window, const float* __restrict__ partials, int max_blocks) {
+                      int head_dim, int window, const float* __restrict__ partials, int max_blocks, int chunk,
+                      const float* __restrict__ sinks) {  // (head_dim: the values' head size)
   const int t = blockIdx.x;
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   const int h = blockIdx.y * kWavesPerBlock + wave;
   if (h >= n_q_heads) return;
   const int p = positions[t];
-  const int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  const int lo = first_key(p, window, chunk);
   const int n_blocks = (p - (lo - lo % kWave)) / kWave + 1;
   const int stride = head_dim + kPartialExtra;
   const float* src = partials + ((size_t)t * n_q_heads + h) * max_blocks * stride;
@@ -449,7 +476,7 @@ attention_join_kernel(T* __restrict__ out, int out_stride, const int32_t* __rest
       if (r0 + u < n_blocks) merge_block(m, l, acc, m_b[u], l_b[u], o_b[u]);
   }
   T* o = out + (size_t)t * out_stride + (size_t)h * head_dim;
-  const float inv_l = 1.0f / l;
+  const float inv_l = 1.0f / with_sink(l, m, sinks, h);
 #pragma unroll
   for (int c = 0; c < kChanPerLane; ++c) {
     const int d = lane + c * kWave;
@@ -466,25 +493,27 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
                                    const void* k_pages, const void* v_pages, const int32_t* token_seq,
                                    const int32_t* positions, const int32_t* block_table, int bt_stride,
                                    int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
-                                   int page_size, int window, float scale, int dtype,
-                                   hipStream_t stream) {
+                                   int page_size, int window, float scale, float softcap, int chunk,
+                                   const float* sinks, int v_dim, int dtype, hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q_heads > 0 && n_kv_heads > 0 && page_size > 0 && bt_stride > 0,
              "attention: bad sizes");
   TL_REQUIRE(n_q_heads % n_kv_heads == 0, "attention: %d query heads are not a multiple of %d kv heads",
              n_q_heads, n_kv_heads);
   if (head_dim <= 0 || head_dim > kMaxHeadDim)
     return tl_fail(TL_ERR_UNSUPPORTED, "attention: head_dim=%d outside 1..%d", head_dim, kMaxHeadDim);
-  TL_REQUIRE(window >= 0, "attention: window=%d must be >= 0", window);
+  TL_REQUIRE(window >= 0 && chunk >= 0, "attention: window=%d and chunk=%d must be >= 0", window, chunk);
+  if (v_dim <= 0 || v_dim > kMaxHeadDim)
+    return tl_fail(TL_ERR_UNSUPPORTED, "attention: values of head size %d outside 1..%d", v_dim, kMaxHeadDim);
   if (n_tokens == 0) return TL_OK;
   dim3 grid(n_tokens, (n_q_heads + kWavesPerBlock - 1) / kWavesPerBlock);
   // rows of the pages start at multiples of head_dim elements from an allocation's start
-  const bool vec = head_dim % 4 == 0 && ((uintptr_t)k_pages % 16) == 0;
+  const bool vec = head_dim % 4 == 0 && v_dim % 4 == 0 && ((uintptr_t)k_pages % 16) == 0 && ((uintptr_t)v_pages % 16) == 0;
   // prompt portions: tokens and heads that read the same keys share them through LDS (same bits)
   if (n_tokens >= kTileMinTokens) {
     const int group = n_q_heads / n_kv_heads;
     const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
     const int qt = kTileWaves / hb;
-    const size_t lds = ((size_t)kTileWaves * head_dim + 2 * (size_t)kWave * (head_dim + kTilePad)) * sizeof(float);
+    const size_t lds = ((size_t)kTileWaves * head_dim + (size_t)kWave * (head_dim + v_dim + 2 * kTilePad)) * sizeof(float);
     dim3 tgrid((n_tokens + qt - 1) / qt, (n_q_heads + hb - 1) / hb);
 #define TL_TILE_LAUNCH_CH(T, VEC, CH)                                                                            \
   do {                                                                                                           \
@@ -495,13 +524,14 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
     }                                                                                                            \
     attention_tile_kernel<T, VEC, CH><<<tgrid, kTileWaves * kWave, lds, stream>>>(                               \
         (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions,  \
-        block_table, bt_stride, n_tokens, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, hb);        \
+        block_table, bt_stride, n_tokens, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, hb, softcap, \
+        chunk, sinks, v_dim);                                                                                    \
   } while (0)
 #define TL_TILE_LAUNCH(T, VEC)                                                                                   \
   do {                                                                                                           \
-    if (head_dim <= 64) TL_TILE_LAUNCH_CH(T, VEC, 1);                                                            \
-    else if (head_dim <= 128) TL_TILE_LAUNCH_CH(T, VEC, 2);                                                      \
-    else if (head_dim <= 192) TL_TILE_LAUNCH_CH(T, VEC, 3);                                                      \
+    if (v_dim <= 64) TL_TILE_LAUNCH_CH(T, VEC, 1);                                                               \
+    else if (v_dim <= 128) TL_TILE_LAUNCH_CH(T, VEC, 2);                                                         \
+    else if (v_dim <= 192) TL_TILE_LAUNCH_CH(T, VEC, 3);                                                         \
     else TL_TILE_LAUNCH_CH(T, VEC, 4);                                                                           \
   } while (0)
     if (dtype == TL_F32) {
@@ -520,7 +550,7 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
 #define TL_ATTN_LAUNCH(T, VEC)                                                                              \
   attention_generic_kernel<T, VEC><<<grid, kWavesPerBlock * kWave, 0, stream>>>(                            \
       (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions, \
-      block_table, bt_stride, n_q_heads, n_kv_heads, head_dim, page_size, window, scale)
+      block_table, bt_stride, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, sinks, v_dim)
   if (dtype == TL_F32) {
     if (vec) TL_ATTN_LAUNCH(float, true);
     else TL_ATTN_LAUNCH(float, false);
@@ -542,7 +572,8 @@ TL_EXPORT int tl_attention_generic_split(const void* q, int q_stride, void* out,
                                          const void* k_pages, const void* v_pages, const int32_t* token_seq,
                                          const int32_t* positions, const int32_t* block_table, int bt_stride,
                                          int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
-                                         int page_size, int window, float scale, int dtype, int max_blocks,
+                                         int page_size, int window, float scale, float softcap, int chunk,
+                                         const float* sinks, int v_dim, int dtype, int max_blocks,
                                          float* partials, hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q_heads > 0 && n_kv_heads > 0 && page_size > 0 && bt_stride > 0,
              "attention: bad sizes");
@@ -550,23 +581,25 @@ TL_EXPORT int tl_attention_generic_split(const void* q, int q_stride, void* out,
              n_q_heads, n_kv_heads);
   if (head_dim <= 0 || head_dim > kMaxHeadDim)
     return tl_fail(TL_ERR_UNSUPPORTED, "attention: head_dim=%d outside 1..%d", head_dim, kMaxHeadDim);
-  TL_REQUIRE(window >= 0, "attention: window=%d must be >= 0", window);
+  TL_REQUIRE(window >= 0 && chunk >= 0, "attention: window=%d and chunk=%d must be >= 0", window, chunk);
+  if (v_dim <= 0 || v_dim > kMaxHeadDim)
+    return tl_fail(TL_ERR_UNSUPPORTED, "attention: values of head size %d outside 1..%d", v_dim, kMaxHeadDim);
   TL_REQUIRE(max_blocks >= 1 && max_blocks <= 65535 && partials != nullptr, "attention: max_blocks=%d outside 1..65535, or no workspace", max_blocks);
   TL_REQUIRE(n_tokens <= 65535, "attention: the split form takes at most 65535 tokens");
   if (n_tokens == 0) return TL_OK;
   const int head_blocks = (n_q_heads + kWavesPerBlock - 1) / kWavesPerBlock;
   dim3 grid(n_tokens, head_blocks, max_blocks);
   dim3 grid_join(n_tokens, head_blocks);
-  const bool vec = head_dim % 4 == 0 && ((uintptr_t)k_pages % 16) == 0;
+  const bool vec = head_dim % 4 == 0 && v_dim % 4 == 0 && ((uintptr_t)k_pages % 16) == 0 && ((uintptr_t)v_pages % 16) == 0;
 #define TL_ATTN_LAUNCH(T, VEC)                                                                                  \
   do {                                                                                                          \
     attention_blocks_kernel<T, VEC><<<grid, kWavesPerBlock * kWave, 0, stream>>>(                               \
         (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions, block_table, bt_stride, \
-        n_q_heads, n_kv_heads, head_dim, page_size, window, scale, partials, max_blocks);                       \
+        n_q_heads, n_kv_heads, head_dim, page_size, window, scale, partials, max_blocks, softcap, chunk, v_dim); \
     int rc = tl_check_launch("attention_blocks");                                                               \
     if (rc != TL_OK) return rc;                                                                                 \
     attention_join_kernel<T><<<grid_join, kWavesPerBlock * kWave, 0, stream>>>(                                 \
-        (T*)out, out_stride, positions, n_q_heads, head_dim, window, partials, max_blocks);                     \
+        (T*)out, out_stride, positions, n_q_heads, v_dim, window, partials, max_blocks, chunk, sinks);         \
   } while (0)
   if (dtype == TL_F32) {
     if (vec) TL_ATTN_LAUNCH(float, true);

@@ -31,7 +31,7 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens live requests hold at any time (each request rounded up to 64)")
     p.add_argument("--page-size", type=int, default=16, help="tokens per cache page (default 16)")
-    p.add_argument("--max-seqs", type=int, default=8, help="request slots (default 8)")
+    p.add_argument("--max-seqs", type=int, default=4, help="request slots (default 4)")
     p.add_argument("--kernel-table", default=None,
                    help="JSON file of matrix-product kernel choices (bfloat16): read if it exists, so that this run uses "
                         "the kernels of the run that wrote it and rounds as that run did; else written after the "

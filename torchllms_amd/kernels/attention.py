@@ -26,15 +26,24 @@ def paged_attention(
     group: int,
     window: int,
     scale: float,
+    softcap: float = 0.0,
+    chunk: int = 0,
+    sinks=None,
+    v_head_dim=None,
 ) -> torch.Tensor:
     """Attention of this step's queries (first Hq * dh columns of ``qkv``) over their requests'
-    cached keys and values; returns [n_tokens, Hq * dh]."""
+    cached keys and values; returns [n_tokens, Hq * dv].  Capped scores (``softcap``), chunks
+    (``chunk``), sinks and values of another head size than the keys are the plain kernel's alone."""
     n = qkv.shape[0]
     n_dec = ctx.host.n_decode
-    fast_decode = n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
+    v_dim = head_dim if v_head_dim is None else int(v_head_dim)
+    plain_only = softcap > 0 or chunk > 0 or sinks is not None or v_dim != head_dim
+    extras = dict(softcap=softcap, chunk=chunk, sinks=sinks, v_head_dim=v_dim) if plain_only else {}
+    fast_decode = not plain_only and n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
     # the MFMA prefill kernel takes positive softmax scales only; anything else runs the plain kernel
-    fast_prefill = n_dec < n and scale > 0 and ops.prefill_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim, k_pages.shape[2])
-    out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+    fast_prefill = (not plain_only and n_dec < n and scale > 0
+                    and ops.prefill_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim, k_pages.shape[2]))
+    out = torch.empty((n, n_q_heads * v_dim), dtype=qkv.dtype, device=qkv.device)
     # rows with a single new token come first in the batch
     if n_dec > 0:
         if ctx.decode_longest is not None:
@@ -56,11 +65,13 @@ def paged_attention(
             # blocks of 64 keys get waves of their own (the same bits either way)
             if window > 0:
                 longest = min(longest, window)
+            if chunk > 0:
+                longest = min(longest, chunk)
             plain = ops.attention_generic_split if longest > GENERIC_SPLIT_FROM else ops.attention_generic
             extra = dict(longest=longest) if longest > GENERIC_SPLIT_FROM else {}
             plain(
                 qkv[:n_dec], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[:n_dec],
-                ctx.positions[:n_dec], ctx.block_tables[group], window, scale, out=out[:n_dec], **extra,
+                ctx.positions[:n_dec], ctx.block_tables[group], window, scale, out=out[:n_dec], **extra, **extras,
             )
     # rows that bring a portion of a prompt take the tiled MFMA kernel
     if n_dec < n:
@@ -85,6 +96,6 @@ def paged_attention(
         else:
             ops.attention_generic(
                 qkv[n_dec:], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[n_dec:],
-                ctx.positions[n_dec:], ctx.block_tables[group], window, scale, out=out[n_dec:],
+                ctx.positions[n_dec:], ctx.block_tables[group], window, scale, out=out[n_dec:], **extras,
             )
     return out

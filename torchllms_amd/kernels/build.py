@@ -35,6 +35,7 @@ CORE_SOURCES = [
     "gemm_stream.hip",
     "gemm_wide.hip",
     "sampling.hip",
+    "sequence_ops.hip",
 ]
 HEADERS = ["common.h", "qkv_epilogue.h", "no_alloc.h"]
 

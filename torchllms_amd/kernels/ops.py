@@ -9,6 +9,8 @@ a module's own helpers and tables stay in the module.
 ``elementwise_ops``  embedding, RMS norm, rotary + cache write, gate, bias
 ``products``         matrix products and the measurement that picks their kernel
 ``attention_ops``    plain, decode and prefill attention with their launch plans
+``sequence_ops``     layer norm with a scaled sum, gated activations, unit-norm rotation with the cache
+                     write, short convolutions, selective scan, gated delta rule
 ``sampling_ops``     the sampling kernel
 """
 
@@ -85,6 +87,17 @@ from .attention_ops import (  # noqa: F401
     prefill_queries_per_tile,
     prefill_tile_count,
     prefill_tiles,
+)
+from .sequence_ops import (  # noqa: F401
+    ScaledSum,
+    causal_conv,
+    embed_scaled,
+    gated_delta,
+    gelu_mul,
+    layernorm,
+    rope_norm_kv_write,
+    selective_scan,
+    state_region,
 )
 from .sampling_ops import (  # noqa: F401
     philox_uniform,

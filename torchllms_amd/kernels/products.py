@@ -637,10 +637,17 @@ def linear_to_sum(x: torch.Tensor, w: torch.Tensor, may_wait: bool = False):
     return run_choice(choice, x, w, x.dtype, leave_split=True)
 
 
-def linear_glu(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """``silu(x @ gate.T) * (x @ up.T)`` for ``w`` [2F, K] = gate rows | up rows: one fused kernel
-    where one of the decode kernels serves the shape, else the product followed by the gate.  ``x``
-    may be ``NormedRows``: the weight-streaming kernel applies them, for any other they are normed first."""
+def linear_glu(x: torch.Tensor, w: torch.Tensor, activation: str = "silu") -> torch.Tensor:
+    """``act(x @ gate.T) * (x @ up.T)`` for ``w`` [2F, K] = gate rows | up rows.  With silu: one fused
+    kernel where one of the decode kernels serves the shape, else the product followed by the gate.  ``x``
+    may be ``NormedRows``: the weight-streaming kernel applies them, for any other they are normed first.
+    With "gelu_tanh" the product is followed by the gate's kernel."""
+    if activation != "silu":
+        if activation != "gelu_tanh":
+            raise KernelError(f"linear_glu: activation {activation!r} (silu, gelu_tanh)")
+        from .sequence_ops import gelu_mul
+
+        return gelu_mul(linear(resolved(x), w))
     if isinstance(x, NormedRows):
         choice = linear_choice(x.gained, w, "glu")
         if choice is not None and choice[0] == "stream":

@@ -27,7 +27,12 @@ class Attention(Mixer):
     limits a query at position p to keys p-w+1..p.  ``shares_kv``: this layer has no k/v
     projections and reads the cache of the run named by the execution order.  ``kv_page_size``:
     tokens per page of this layer's keys and values, when not the engine's own (layers that ask for
-    the same form a group of pages of their own).
+    the same form a group of pages of their own).  ``v_head_dim``: the values' head size when it is
+    not the keys'.  ``qk_norm_eps`` > 0: after the rotation every query and key head is divided by its
+    root mean square (eps under the root, no weight).  ``softcap`` c > 0: scores become
+    c tanh(score / c).  ``chunk`` n > 0: a query sees only the keys of its own chunk of n positions,
+    chunks counted from position 0.  ``sinks``: a learned number per query head (tensor ``sinks``)
+    whose exponential joins the softmax's denominator, with no value behind it.
     """
 
     #: every launch is fixed by the step's shape: a decode step may be recorded in a HIP graph
@@ -46,6 +51,11 @@ class Attention(Mixer):
         position: PartSpec,
         shares_kv: bool = False,
         kv_page_size: Optional[int] = None,
+        v_head_dim: Optional[int] = None,
+        qk_norm_eps: float = 0.0,
+        softcap: float = 0.0,
+        chunk: int = 0,
+        sinks: bool = False,
     ):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
@@ -58,18 +68,36 @@ class Attention(Mixer):
         self.window = int(window)
         self.shares_kv = shares_kv
         self.kv_page_size = kv_page_size
+        self.v_head_dim = int(v_head_dim) if v_head_dim else head_dim
+        self.qk_norm_eps = float(qk_norm_eps)
+        self.softcap = float(softcap)
+        self.chunk = int(chunk)
+        self.has_sinks = bool(sinks)
+        if self.qk_norm_eps < 0 or self.softcap < 0 or self.chunk < 0:
+            raise ValueError("attention: qk_norm_eps, softcap and chunk must not be negative")
+        if qkv_bias and self.extended:
+            raise ValueError("attention: q/k/v biases together with a unit norm, capped scores, chunks, sinks or values of their own size are not built")
+        self.sinks: Optional[torch.Tensor] = None
         self.position = POSITIONS.build(position)
         self.wqkv: Optional[torch.Tensor] = None
         self.bqkv: Optional[torch.Tensor] = None
         self.wo: Optional[torch.Tensor] = None
 
+    @property
+    def extended(self) -> bool:
+        """Whether the layer needs what only the unfused path and the plain attention kernel do."""
+        return (self.v_head_dim != self.head_dim or self.qk_norm_eps > 0 or self.softcap > 0 or self.chunk > 0 or self.has_sinks)
+
     def param_specs(self) -> Dict[str, ParamSpec]:
         q = self.num_heads * self.head_dim
         kv = self.num_kv_heads * self.head_dim
-        specs = {"wq.weight": ParamSpec((q, self.hidden_size)), "wo.weight": ParamSpec((self.hidden_size, q))}
+        specs = {"wq.weight": ParamSpec((q, self.hidden_size)),
+                 "wo.weight": ParamSpec((self.hidden_size, self.num_heads * self.v_head_dim))}
         if not self.shares_kv:
             specs["wk.weight"] = ParamSpec((kv, self.hidden_size))
-            specs["wv.weight"] = ParamSpec((kv, self.hidden_size))
+            specs["wv.weight"] = ParamSpec((self.num_kv_heads * self.v_head_dim, self.hidden_size))
+        if self.has_sinks:
+            specs["sinks"] = ParamSpec((self.num_heads,), kind="vector", init="zeros")
         if self.qkv_bias:
             specs["wq.bias"] = ParamSpec((q,), init="zeros")
             if not self.shares_kv:
@@ -78,12 +106,14 @@ class Attention(Mixer):
         return specs
 
     def check_sizes(self, dtype: torch.dtype) -> None:
+        if not 0 < self.v_head_dim <= ops.ATTENTION_MAX_HEAD_DIM:
+            raise ValueError(f"attention: values of head size {self.v_head_dim}; the attention kernels take up to {ops.ATTENTION_MAX_HEAD_DIM}")
         if not 0 < self.head_dim <= ops.ATTENTION_MAX_HEAD_DIM:
             raise ValueError(
                 f"attention: head size {self.head_dim}; the attention kernels take head sizes up to "
                 f"{ops.ATTENTION_MAX_HEAD_DIM} (any number of heads and of query heads per kv head)"
             )
-        if dtype == torch.bfloat16:
+        if dtype == torch.bfloat16 and not self.extended:
             fast = (ops.decode_attention_supported(dtype, self.num_heads, self.num_kv_heads, self.head_dim),
                     ops.prefill_attention_supported(dtype, self.num_heads, self.num_kv_heads, self.head_dim))
             said = (self.num_heads, self.num_kv_heads, self.head_dim)
@@ -102,7 +132,8 @@ class Attention(Mixer):
     def cache_need(self):
         if self.shares_kv:
             return None
-        return KVNeed(num_kv_heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window, page_size=self.kv_page_size)
+        return KVNeed(num_kv_heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window, page_size=self.kv_page_size,
+                      v_head_dim=self.v_head_dim if self.v_head_dim != self.head_dim else None)
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         names = ["wq"] if self.shares_kv else ["wq", "wk", "wv"]
@@ -111,6 +142,8 @@ class Attention(Mixer):
         if self.qkv_bias:
             self.bqkv = torch.cat([tensors[f"{n}.bias"] for n in names], dim=0).contiguous()
         self.wo = tensors["wo.weight"].contiguous()
+        if self.has_sinks:
+            self.sinks = tensors["sinks"].float().contiguous()
         self.position.to(self.wo.device)
 
     def linear_weights(self):
@@ -129,6 +162,8 @@ class Attention(Mixer):
             table = ctx.scratch.get(key)
             if table is None:
                 table = ctx.scratch[key] = ops.rope_table(ctx.positions, rot.inv_freq)
+        if self.extended:
+            return self._forward_extended(x, ctx, cache, n_kv_in_row, rot, table, store)
         qkv = ops.qkv_rope_store(
             x,
             self.wqkv,
@@ -149,5 +184,23 @@ class Attention(Mixer):
         attn = paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
             ctx, g, self.window, self.softmax_scale,
+        )
+        return ops.linear_to_sum(attn, self.wo, may_wait=True)
+
+    def _forward_extended(self, x, ctx, cache, n_kv_in_row, rot, table, store):
+        """The layer with a unit norm on queries and keys, capped scores, chunks, sinks or values of their
+        own head size: the projection, then rotation, norm and cache write in one kernel, then the plain
+        attention kernel, which takes all of these."""
+        g = cache.group
+        qkv = ops.linear(ops.resolved(x), self.wqkv)
+        ops.rope_norm_kv_write(
+            qkv, self.num_heads, n_kv_in_row, self.head_dim, self.v_head_dim, table, rot.rotary_dim if rot else 0,
+            rot.pairing if rot else 0, self.qk_norm_eps,
+            cache.k_pages if store else None, cache.v_pages if store else None,
+            ctx.slot_mappings[g] if store else None, cache.page_size if store else 0,
+        )
+        attn = paged_attention(
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages, ctx, g, self.window,
+            self.softmax_scale, softcap=self.softcap, chunk=self.chunk, sinks=self.sinks, v_head_dim=self.v_head_dim,
         )
         return ops.linear_to_sum(attn, self.wo, may_wait=True)

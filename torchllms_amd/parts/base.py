@@ -33,7 +33,8 @@ class ParamSpec:
 
     ``kind``: "matrix" (kept in the model's compute dtype), "vector" (compute dtype, but a
     tensor stored in 32-bit stays in 32-bit), "int" (an integer table, kept as int32).
-    ``init``: how the random-weights mode fills it: "normal" N(0, 0.02), "ones", "zeros".
+    ``init``: how the random-weights mode fills it: "normal" N(0, 0.02), "ones", "zeros", "conv" and "wide" (N(0, 0.5):
+    the taps of a short convolution, a projection from very few inputs).
     """
 
     shape: Tuple[int, ...]
@@ -49,6 +50,7 @@ class KVNeed:
     sees positions p-w+1 .. p only, so pages that lie wholly before that may be given back.
     ``page_size`` (tokens per page) and ``dtype`` ("float32", "bfloat16") are the engine's own
     unless the mixer asks for others; layers that ask for the same form one group of pages.
+    ``v_head_dim``: the head size of the values when it is not that of the keys.
     """
 
     num_kv_heads: int
@@ -56,6 +58,7 @@ class KVNeed:
     window: int = 0
     page_size: Optional[int] = None
     dtype: Optional[str] = None
+    v_head_dim: Optional[int] = None
 
 
 @dataclass(frozen=True)

@@ -12,13 +12,21 @@ from .base import EMBEDDINGS, HEADS, Embedding, Head, ParamSpec
 
 @EMBEDDINGS.register("embedding")
 class TokenEmbedding(Embedding):
-    """``h = weight[token]``, no scale factor (reference: torchllms/models/networks.py:793,1017)."""
+    """``h = weight[token]`` (reference: torchllms/models/networks.py:793,1017, which has no scale
+    factor).  ``stream_dtype`` "float32": the rows open a 32-bit residual stream whatever the model's
+    dtype, as ``float(weight[token]) * scale``."""
 
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, stream_dtype: Optional[str] = None):
+        if stream_dtype not in (None, "float32"):
+            raise ValueError(f"embedding: stream_dtype {stream_dtype!r} (None: the model's dtype, or \"float32\")")
+        if stream_dtype is None and float(scale) != 1.0:
+            raise ValueError("embedding: a scale factor needs the 32-bit residual stream (stream_dtype=\"float32\")")
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
+        self.scale = float(scale)
+        self.stream_dtype = stream_dtype
         self.weight: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -28,6 +36,8 @@ class TokenEmbedding(Embedding):
         self.weight = tensors["weight"].contiguous()
 
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        if self.stream_dtype == "float32":
+            return ops.embed_scaled(tokens, self.weight, self.scale)
         return ops.embed(tokens, self.weight)
 
 

@@ -12,13 +12,16 @@ from .base import FEED_FORWARDS, FeedForward, ParamSpec
 
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
-    """``w2( silu(w1 x) * (w3 x) )`` without biases
-    (reference: torchllms/models/networks.py:592-605)."""
+    """``w2( act(w1 x) * (w3 x) )`` without biases, act = silu
+    (reference: torchllms/models/networks.py:592-605) or, with ``activation="gelu_tanh"``, the tanh form of gelu."""
 
     graph_safe = True
     takes_normed_rows = True
 
-    def __init__(self, hidden_size: int, intermediate_size: int):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+        if activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"gated feed-forward: activation {activation!r} (silu, gelu_tanh)")
+        self.activation = activation
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.w13: Optional[torch.Tensor] = None
@@ -34,7 +37,8 @@ class SwiGLU(FeedForward):
         self.w2 = tensors["w2.weight"].contiguous()
 
     def linear_weights(self):
-        return [(self.w13, "glu"), (self.w2, "sum")]
+        # (only the silu gate has fused forms; another activation runs the plain product and then the gate)
+        return [(self.w13, "glu" if self.activation == "silu" else "plain"), (self.w2, "sum")]
 
     def forward(self, x, ctx):
-        return ops.linear_to_sum(ops.linear_glu(x, self.w13), self.w2, may_wait=True)
+        return ops.linear_to_sum(ops.linear_glu(x, self.w13, self.activation), self.w2, may_wait=True)

@@ -16,6 +16,7 @@ from . import embedding as _embedding  # noqa: F401
 from . import feed_forward as _feed_forward  # noqa: F401
 from . import norms as _norms  # noqa: F401
 from . import positions as _positions  # noqa: F401
+from . import recurrent as _recurrent  # noqa: F401
 
 
 class Model:

@@ -50,3 +50,49 @@ class RMSNorm(Norm):
 
     def forward_rows(self, h: torch.Tensor, delta: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
         return ops.rmsnorm(h, self.weight, self.eps, delta=delta, rows=rows)
+
+
+@NORMS.register("layernorm")
+class LayerNorm(Norm):
+    """``y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight + bias``, statistics in 32-bit.  The
+    residual stream it reads may be 32-bit in a bfloat16 model; what it hands on has the model's dtype.
+    Its kernel adds a ``ScaledSum`` (a factor times the sum of a layer's branches) to the stream on the way."""
+
+    graph_safe = True
+
+    def __init__(self, size: int, eps: float):
+        self.size = size
+        self.eps = float(eps)
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+        self.out_dtype: Optional[torch.dtype] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        # (kind "matrix": the vectors follow the model's dtype, which is the dtype of the normed rows)
+        return {"weight": ParamSpec((self.size,), kind="matrix", init="ones"), "bias": ParamSpec((self.size,), kind="matrix", init="zeros")}
+
+    def check_sizes(self, dtype: torch.dtype) -> None:
+        if not 0 < self.size <= ops.rmsnorm_max_hidden():
+            raise ValueError(f"layernorm: rows of {self.size} elements; the kernel takes 1 to {ops.rmsnorm_max_hidden()}")
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.out_dtype = tensors["weight"].dtype
+        self.weight = tensors["weight"].float().contiguous()
+        self.bias = tensors["bias"].float().contiguous()
+
+    def delta(self, delta):
+        if delta is None or isinstance(delta, ops.ScaledSum):
+            return delta
+        return ops.ScaledSum([ops.resolved(delta)], 1.0)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.layernorm(x, self.weight, self.bias, self.eps, self.out_dtype)
+
+    def forward_add(self, h: torch.Tensor, delta):
+        delta = self.delta(delta)
+        if delta is None:
+            return h, ops.layernorm(h, self.weight, self.bias, self.eps, self.out_dtype)
+        return ops.layernorm(h, self.weight, self.bias, self.eps, self.out_dtype, delta=delta, return_sum=True)
+
+    def forward_rows(self, h: torch.Tensor, delta, rows: torch.Tensor) -> torch.Tensor:
+        return ops.layernorm(h, self.weight, self.bias, self.eps, self.out_dtype, delta=self.delta(delta), rows=rows)

@@ -122,3 +122,36 @@ def llama_name_rules(cfg) -> List[NameRule]:
         NameRule("output.weight", "head.weight"),
     ]
     return rules
+
+
+def taluvik_name_rules(cfg) -> List[NameRule]:
+    """Taluvik checkpoints name a layer's tensors ``l<i>.norm1[.b]``, ``l<i>.mix.<tensor>`` and
+    ``l<i>.mlp.{gate,up,down}``; the parts' own names differ only where a part is shared with other
+    architectures (the norm, the attention, the gated feed-forward)."""
+    L = "l{}."
+    rules = [
+        NameRule("embed", "embed.weight"),
+        NameRule("final.norm", "final_norm.weight"),
+        NameRule("final.norm.b", "final_norm.bias"),
+        NameRule("head", "head.weight"),
+        NameRule(L + "norm1", L + "norm1.weight"),
+        NameRule(L + "norm1.b", L + "norm1.bias"),
+        NameRule(L + "mlp.gate", L + "mlp.w1.weight"),
+        NameRule(L + "mlp.up", L + "mlp.w3.weight"),
+        NameRule(L + "mlp.down", L + "mlp.w2.weight"),
+    ]
+    kinds = {layer.type for layer in cfg.layers}
+    attention = {"q": "wq.weight", "k": "wk.weight", "v": "wv.weight", "o": "wo.weight", "sink": "sinks"}
+    recurrent = ["in", "conv", "conv.b", "x", "dt", "dt.b", "A_log", "D", "o", "q", "q.conv", "k", "k.conv", "v", "v.conv",
+                 "b", "a", "dt_bias", "norm", "g"]
+    # a tensor's name alone does not say which mixer it belongs to (every mixer has an "o"): the rules are
+    # written per layer, from the layer's type
+    for i, layer in enumerate(cfg.layers):
+        if layer.weights_of is not None:
+            continue
+        p = f"l{i}.mix."
+        if layer.type == "attention":
+            rules += [NameRule(p + ext, p + own) for ext, own in attention.items()]
+        else:
+            rules += [NameRule(p + n, p + n) for n in recurrent]
+    return rules

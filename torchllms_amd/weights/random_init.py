@@ -41,6 +41,12 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, dtype: torch.dtype, nor
         t = torch.ones(spec.shape, dtype=torch.float32, device=device)
         if norm_jitter > 0:
             t += torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, norm_jitter, generator=gen)
+    elif spec.init == "conv":
+        # taps of a short convolution: of the order of one over their number, so that signals pass
+        t = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, 0.5, generator=gen)
+    elif spec.init == "wide":
+        # a projection from very few inputs (a low-rank step size): N(0, 0.02) would leave it flat
+        t = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, 0.5, generator=gen)
     elif spec.init == "zeros":
         t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
         if norm_jitter > 0:
@@ -112,10 +118,9 @@ def main(argv=None) -> int:
         path = path / "config.json"
     with open(path) as f:
         raw = json.load(f)
-    names = raw.get("architectures") or []
-    if not names:
-        raise SystemExit(f"{path} names no architecture (key \"architectures\")")
-    arch = get_architecture(names[0])
+    from ..config.registry import architecture_name
+
+    arch = get_architecture(architecture_name(raw))
     config = arch.config_from_dict(raw)
     dtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
     folder = write_model_folder(args.out, config, args.seed, dtype=dtype, norm_jitter=args.norm_jitter, arch=arch)
