@@ -50,11 +50,10 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor
     S, C = x.shape
     K = taps.shape[1]
     out = torch.zeros_like(x)
-    for t in range(S):
-        for j in range(K):
-            src = t - (K - 1 - j)
-            if src >= 0:
-                out[t] += taps[:, j] * x[src]
+    for j in range(K):
+        back = K - 1 - j  # how many tokens before the current one column j reads
+        if back < S:
+            out[back:] += taps[:, j] * x[: S - back]
     if bias is not None:
         out = out + bias
     return out
@@ -98,18 +97,15 @@ def attention_scores_to_output(q, k, v, scale, softcap, chunk, sink, positions):
     """q [S, d], k [S, d], v [S, dv] of one head; ``positions`` [S] absolute.  Token i reads token
     j <= i of its own chunk of ``chunk`` positions; the softmax has one more term exp(sink) in its
     denominator that carries no value."""
-    S = q.shape[0]
-    out = torch.zeros((S, v.shape[1]), dtype=q.dtype)
-    for i in range(S):
-        pi = int(positions[i])
-        js = [j for j in range(i + 1) if int(positions[j]) // chunk == pi // chunk]
-        s = (k[js] @ q[i]) * scale
-        s = softcap * torch.tanh(s / softcap)
-        m = max(float(s.max()), float(sink))
-        e = torch.exp(s - m)
-        denom = e.sum() + math.exp(float(sink) - m)
-        out[i] = (e / denom) @ v[js]
-    return out
+    s = (q @ k.T) * scale
+    s = softcap * torch.tanh(s / softcap)
+    pi, pj = positions[:, None], positions[None, :]
+    seen = (pj <= pi) & (torch.div(pj, chunk, rounding_mode="floor") == torch.div(pi, chunk, rounding_mode="floor"))
+    s = s.masked_fill(~seen, float("-inf"))
+    m = torch.clamp(s.max(dim=-1, keepdim=True).values, min=float(sink))
+    e = torch.exp(s - m)
+    denom = e.sum(dim=-1, keepdim=True) + torch.exp(sink - m)
+    return (e / denom) @ v
 
 
 def attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: dict, eps: float,
@@ -142,15 +138,15 @@ def delta_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: dict, ep
     beta = torch.sigmoid(h @ w[p + "b"].T)  # [S, H]
     decay = torch.exp(-torch.exp(w[p + "A_log"]) * softplus(h @ w[p + "a"].T + w[p + "dt_bias"]))  # [S, H]
     gate = silu(h @ w[p + "g"].T).view(S, H, dv)
+    rep = H // G  # head h reads q/k head h // rep
+    qh, kh = q.repeat_interleave(rep, dim=1), k.repeat_interleave(rep, dim=1)  # [S, H, d]
     out = torch.zeros((S, H, dv), dtype=h.dtype)
-    for head in range(H):
-        g = head // (H // G)
-        state = torch.zeros((d, dv), dtype=h.dtype)
-        for t in range(S):
-            state = decay[t, head] * state
-            u = beta[t, head] * (v[t, head] - state.T @ k[t, g])
-            state = state + torch.outer(k[t, g], u)
-            out[t, head] = state.T @ q[t, g]
+    state = torch.zeros((H, d, dv), dtype=h.dtype)
+    for t in range(S):
+        state = decay[t][:, None, None] * state
+        u = beta[t][:, None] * (v[t] - torch.einsum("hij,hi->hj", state, kh[t]))
+        state = state + torch.einsum("hi,hj->hij", kh[t], u)
+        out[t] = torch.einsum("hij,hi->hj", state, qh[t])
     out = rms_unit(out, eps) * w[p + "norm"] * gate
     return out.reshape(S, H * dv) @ w[p + "o"].T
 

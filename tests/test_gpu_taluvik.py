@@ -1,0 +1,344 @@
+"""The Taluvik decoder in the engine against the plain implementation of tests/plain/taluvik.py:
+every mechanism alone, whole prompts against decoding token by token, portions down to two tokens,
+mixed batches with pages and state slots that are used again, long decoding from recorded graphs,
+and greedy generation through ``LLM.generate`` and the scheduler; on three small configurations that
+differ in every size, in 32-bit and in bfloat16."""
+
+import math
+
+import pytest
+import torch
+
+from . import schedules
+from . import taluvik_models as models
+from .helpers import random_tokens
+from .plain import taluvik as plain
+from .test_gpu_engine import run_trace
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [70, 41, 100, 35, 50, 33], "B": [66, 40, 130, 35, 90], "C": [45, 150, 37, 64, 120]}
+#: distances are measured as the checker of a replay would: the difference of two rows of logits with
+#: its mean taken off, root mean square over the vocabulary, over the root mean square of the truth
+FP32_TOL = 2e-5
+BF16_TOL = 4e-2
+
+
+def distance(got: torch.Tensor, truth: torch.Tensor, scale: float) -> float:
+    d = got.double() - truth.double()
+    d = d - d.mean()
+    return float(d.pow(2).mean().sqrt()) / scale
+
+
+def truth_of(cfg, weights, requests):
+    w64 = {k: v.double() for k, v in weights.items()}
+    out = {rid: plain.forward(cfg, w64, toks) for rid, toks in requests.items()}
+    scale = float(torch.cat([(t - t.mean(-1, keepdim=True)).flatten() for t in out.values()]).pow(2).mean().sqrt())
+    return out, scale
+
+
+class Case:
+    def __init__(self, name, tmp):
+        from torchllms_amd.engine import Engine
+
+        self.name = name
+        self.folder = models.make_folder(tmp / name, models.CONFIGS[name], seed=11)
+        self.cfg, self.weights = models.read_folder(self.folder)
+        self.requests = {f"r{i}": random_tokens(n, self.cfg["vocab"], 100 + i) for i, n in enumerate(LENGTHS[name])}
+        self.truth, self.scale = truth_of(self.cfg, self.weights, self.requests)
+        self.traces = {
+            "whole": schedules.whole(self.requests),
+            "tail": schedules.tail(self.requests),
+            "portions": schedules.portions(self.requests),
+            "mixed": schedules.mixed(self.requests),
+        }
+        page = models.PAGE_SIZE[name]
+        pool_tokens = max(schedules.max_live_tokens(t) for t in self.traces.values())
+        self.engines = {
+            dt: Engine.from_folder(self.folder, dtype=dt, page_size=page, num_pages=-(-pool_tokens // page), max_seqs=4)
+            for dt in ("float32", "bfloat16")
+        }
+        self._results = {}
+
+    def result(self, dtype, schedule):
+        key = (dtype, schedule)
+        if key not in self._results:
+            self._results[key] = run_trace(self.engines[dtype], self.traces[schedule])
+        return self._results[key]
+
+    def worst(self, result):
+        worst, where = 0.0, None
+        for (rid, pos), row in result.items():
+            e = distance(row, self.truth[rid][pos], self.scale)
+            if not e <= worst:
+                worst, where = e, (rid, pos)
+        return worst, where
+
+
+@pytest.fixture(scope="module")
+def cases(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("taluvik")
+    return {name: Case(name, tmp) for name in models.CONFIGS}
+
+
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_float32_matches_the_plain_model(cases, name, schedule):
+    case = cases[name]
+    got = case.result("float32", schedule)
+    assert len(got) == sum(len(t) for t in case.requests.values())
+    err, where = case.worst(got)
+    assert err < FP32_TOL, f"{name}/{schedule}: first look at {where}, distance {err}"
+
+
+@pytest.mark.parametrize("schedule", ["tail", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_float32_does_not_depend_on_the_schedule(cases, name, schedule):
+    """Every 32-bit kernel adds in an order fixed by the element it computes (the recurrences token by
+    token, the attention block by block of 64 keys), so cutting, batching, pages and slots change no bit."""
+    case = cases[name]
+    ref = case.result("float32", "whole")
+    got = case.result("float32", schedule)
+    diff = sorted(k for k in ref if not torch.equal(ref[k], got[k]))
+    assert not diff, f"{name}/{schedule}: {len(diff)} positions differ, first {diff[0]}"
+
+
+@pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_bfloat16_stays_within_rounding(cases, name, schedule):
+    case = cases[name]
+    got = case.result("bfloat16", schedule)
+    err, where = case.worst(got)
+    assert err < BF16_TOL, f"{name}/{schedule}: first look at {where}, distance {err}"
+    mean = sum(distance(row, case.truth[rid][pos], case.scale) for (rid, pos), row in got.items()) / len(got)
+    assert mean < BF16_TOL / 3, f"{name}/{schedule}: mean distance {mean}"
+
+
+# ----------------------------------------------------------------------------- every mechanism alone
+ALONE = {
+    "attention": models.layer("attention", models.attention(4, 2, 32, 48, 20, 16, 0.25, 6.0)),
+    "attention_whole_head_rotated": models.layer("attention", models.attention(3, 3, 16, 16, 16, 9, 0.5, 30.0,
+                                                 scaling={"factor": 4.0, "low": 1.0, "high": 4.0, "original": 16})),
+    "delta": models.layer("delta", {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 40, "conv": 4}),
+    "delta_wide": models.layer("delta", {"heads": 1, "kv_heads": 1, "dim": 256, "vdim": 64, "conv": 2}),
+    "mamba1": models.layer("mamba1", {"inner": 72, "state": 24, "dt_rank": 6, "conv": 3}),
+    "mamba1_many_states": models.layer("mamba1", {"inner": 40, "state": 100, "dt_rank": 8, "conv": 6}),
+    "feed_forward": models.layer("mamba1", {"inner": 8, "state": 1, "dt_rank": 1, "conv": 1}, ff=136),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("what", sorted(ALONE))
+def test_a_mechanism_alone(tmp_path, what, dtype):
+    """A model of one layer with that mixer and no feed-forward (or hardly a mixer and a feed-forward),
+    a prompt in one step and, in a second request, the same tokens in portions and one by one."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    folder = models.make_folder(tmp_path / what, models.single_layer(ALONE[what]), seed=5)
+    cfg, weights = models.read_folder(folder)
+    tokens = random_tokens(75, cfg["vocab"], 9)
+    truth, scale = truth_of(cfg, weights, {"r": tokens})
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=24, max_seqs=2)
+    engine.admit("whole")
+    whole = engine.step([StepEntry("whole", tokens, list(range(len(tokens))))]).cpu()
+    engine.admit("cut")
+    rows, at = [], 0
+    for n in (5, 2, 30, 1, 1, 1, 17, 2, 1, 1, 13, 1):
+        rows.append(engine.step([StepEntry("cut", tokens[at : at + n], list(range(n)))]).cpu())
+        at += n
+    assert at == len(tokens)
+    cut = torch.cat(rows)
+    tol = FP32_TOL if dtype == "float32" else BF16_TOL
+    for name, got in (("whole", whole), ("cut", cut)):
+        worst = max(distance(got[i], truth["r"][i], scale) for i in range(len(tokens)))
+        assert worst < tol, f"{what}/{name}: distance {worst}"
+    if dtype == "float32":
+        assert torch.equal(whole, cut)
+
+
+# ----------------------------------------------------------------------------- attention: edges made visible
+def _paged(keys: torch.Tensor, page_size: int, order):
+    """Keys [n, H, d] into pages [pages, H, page_size, d] handed out in ``order``; returns pages and block table."""
+    n, H, d = keys.shape
+    blocks = -(-n // page_size)
+    pages = torch.zeros((len(order), H, page_size, d), dtype=keys.dtype, device=keys.device)
+    for b in range(blocks):
+        rows = keys[b * page_size : (b + 1) * page_size]
+        pages[order[b], :, : rows.shape[0]] = rows.transpose(0, 1)
+    return pages, torch.tensor([order[:blocks]], dtype=torch.int32, device=keys.device)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("form", ["alone", "tile", "split"])
+def test_one_key_that_stands_out_at_every_edge(form, dtype):
+    """The plain attention kernel with chunks, a cap, sinks and values narrower than keys, on inputs in
+    which one key has a score far above all others.  Queries are placed so that this key is the first of
+    their chunk, the last of the chunk before, at a page's border, far back, or the query itself: the
+    output is that key's value (less the sink's share) or hardly any of it.  All three launches of the kernel."""
+    from torchllms_amd.kernels import ops
+
+    dev = "cuda:0"
+    H, G, d, dv, chunk, page = 4, 2, 32, 16, 48, 16
+    n = 300
+    g = torch.Generator().manual_seed(3)
+    k = torch.randn((n, G, d), generator=g) * 0.3
+    v = torch.randn((n, G, dv), generator=g)
+    special = [0, 47, 48, 95, 96, 143, 144, 160, 239, 240, 287]  # chunk and page borders among them
+    direction = torch.randn(d, generator=g)
+    direction = direction / direction.norm()
+    for j in special:
+        k[j] += 6.0 * direction * (1 + 0.01 * j)
+    sinks = torch.tensor([0.5, -1.0, 2.0, 0.0])
+    scale, cap = 1.3, 9.0
+    if form == "alone":
+        query_at = [0, 1, 46, 47, 48, 49, 94, 95, 96, 97, 143, 144, 159, 160, 161, 239, 240, 241, 286, 287, 288, 299]
+    elif form == "tile":
+        query_at = list(range(n))
+    else:
+        query_at = [299, 287, 241, 240]  # few tokens, each a request of its own length: the split form
+    q = torch.randn((len(query_at), H, d), generator=g) * 0.2 + 4.0 * direction
+    # truth in 64-bit from the formula
+    want = torch.zeros((len(query_at), H, dv), dtype=torch.float64)
+    kd, vd, qd = k.to(dtype).double(), v.to(dtype).double(), q.to(dtype).double()
+    for r, p in enumerate(query_at):
+        lo = p - p % chunk
+        for h in range(H):
+            s = (kd[lo : p + 1, h // 2] @ qd[r, h]) * scale
+            s = cap * torch.tanh(s / cap)
+            m = max(float(s.max()), float(sinks[h]))
+            e = torch.exp(s - m)
+            want[r, h] = (e / (e.sum() + math.exp(float(sinks[h]) - m))) @ vd[lo : p + 1, h // 2]
+    order = torch.randperm(32, generator=g).tolist()
+    k_pages, bt = _paged(k.to(dtype).to(dev), page, order)
+    v_pages, _ = _paged(v.to(dtype).to(dev), page, order)
+    qkv = q.to(dtype).reshape(len(query_at), H * d).to(dev).contiguous()
+    seq = torch.zeros(len(query_at), dtype=torch.int32, device=dev)
+    pos = torch.tensor(query_at, dtype=torch.int32, device=dev)
+    kw = dict(softcap=cap, chunk=chunk, sinks=sinks.to(dev), v_head_dim=dv)
+    if form == "split":
+        got = ops.attention_generic_split(qkv, H, G, d, k_pages, v_pages, seq, pos, bt, 0, scale, longest=chunk, **kw)
+    else:
+        got = ops.attention_generic(qkv, H, G, d, k_pages, v_pages, seq, pos, bt, 0, scale, **kw)
+    got = got.float().cpu().double().reshape(len(query_at), H, dv)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert (got - want).abs().max() < tol, f"first wrong query at position {query_at[int((got - want).abs().amax((1, 2)).argmax())]}"
+    # the inputs do what they are made for: the query right behind a chunk's first key gives nearly all
+    # of its weight to that key, and the query on the chunk's first position cannot see the key before it
+    if 49 in query_at:
+        near = want[query_at.index(49), 1]
+        assert (near - vd[48, 0] * (near @ vd[48, 0]) / (vd[48, 0] @ vd[48, 0])).norm() < 0.2 * near.norm()
+    # the three launches agree bit for bit
+    if form == "tile":
+        few = [0, 47, 48, 49, 143, 144, 299]
+        rows = torch.tensor(few, device=dev)
+        alone = ops.attention_generic(qkv[rows].contiguous(), H, G, d, k_pages, v_pages, seq[: len(few)].contiguous(),
+                                      pos[rows].contiguous(), bt, 0, scale, **kw)
+        split = ops.attention_generic_split(qkv[rows].contiguous(), H, G, d, k_pages, v_pages, seq[: len(few)].contiguous(),
+                                            pos[rows].contiguous(), bt, 0, scale, longest=chunk, **kw)
+        tile = ops.attention_generic(qkv, H, G, d, k_pages, v_pages, seq, pos, bt, 0, scale, **kw)[rows]
+        assert torch.equal(alone, tile) and torch.equal(alone, split)
+
+
+# ----------------------------------------------------------------------------- state that is carried, freed and used again
+def test_slots_and_pages_that_are_used_again_start_clean(tmp_path):
+    """Two slots, few pages: six requests pass through them one after the other and side by side, each
+    beside a neighbour that is at another place of its own sequence; every one must come out as alone."""
+    from torchllms_amd.engine import Engine
+
+    folder = models.make_folder(tmp_path / "m", models.CONFIGS["A"], seed=2)
+    cfg, weights = models.read_folder(folder)
+    requests = {f"q{i}": random_tokens(n, cfg["vocab"], 50 + i) for i, n in enumerate([30, 55, 18, 41, 26, 60])}
+    truth, scale = truth_of(cfg, weights, requests)
+    steps = schedules.mixed(requests, max_live=2)
+    pool = schedules.max_live_tokens(steps, round_to=8)
+    engine = Engine.from_folder(folder, dtype="float32", page_size=8, num_pages=pool // 8, max_seqs=2)
+    got = run_trace(engine, steps)
+    worst = max(distance(row, truth[rid][pos], scale) for (rid, pos), row in got.items())
+    assert worst < FP32_TOL, worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_from_recorded_steps(tmp_path, dtype):
+    """A short prompt and 400 tokens one by one, two requests side by side: the decode steps are
+    recorded as graphs after a few, and replayed; states and histories move on with every replay,
+    chunks begin and end, and the windows of the convolutions hold tokens of the steps before."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    folder = models.make_folder(tmp_path / "m", models.CONFIGS["B"], seed=8)
+    cfg, weights = models.read_folder(folder)
+    requests = {"a": random_tokens(410, cfg["vocab"], 1), "b": random_tokens(425, cfg["vocab"], 2)}
+    truth, scale = truth_of(cfg, weights, requests)
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=64, max_seqs=2)
+    assert engine.graphs is not None
+    heads = {"a": 10, "b": 25}
+    for rid, toks in requests.items():
+        engine.admit(rid)
+        engine.step([StepEntry(rid, toks[: heads[rid]], [])])
+    tol = FP32_TOL if dtype == "float32" else BF16_TOL
+    worst = 0.0
+    for i in range(400):
+        entries = [StepEntry(rid, [requests[rid][heads[rid] + i]], [0]) for rid in ("a", "b")]
+        logits = engine.step(entries).cpu()
+        for row, rid in zip(logits, ("a", "b")):
+            worst = max(worst, distance(row, truth[rid][heads[rid] + i], scale))
+    assert any(g.replays > 100 for g in engine.graphs.graphs.values())
+    assert worst < tol, worst
+
+
+def test_greedy_generation_through_the_entry_point(tmp_path):
+    """``LLM.generate``: the scheduler admits, cuts prompts into portions under a small token budget,
+    decodes everybody together and frees; the tokens are the plain model's."""
+    from torchllms_amd.inference import LLM
+
+    folder = models.make_folder(tmp_path / "m", models.CONFIGS["A"], seed=4)
+    cfg, weights = models.read_folder(folder)
+    w64 = {k: v.double() for k, v in weights.items()}
+    prompts = [random_tokens(n, cfg["vocab"], 40 + n) for n in (5, 37, 1, 64, 22)]
+    new = 20
+
+    def plain_greedy(prompt):
+        toks = list(prompt)
+        for _ in range(new):
+            toks.append(int(plain.forward(cfg, w64, toks)[-1].argmax()))
+        return toks[len(prompt):]
+
+    llm = LLM(str(folder), precision="float32", max_len=128, max_bsz=3, page_size=8, max_num_batched_tokens=24)
+    results = llm.generate(prompt_token_ids=prompts, temperature=0.0, max_new_tokens=new)
+    for p, r in zip(prompts, results):
+        assert r.token_ids == plain_greedy(p)
+    llm.engine.cache.check_invariants()
+    assert llm.engine.cache.live == []
+    # in bfloat16 the first token of each request is the one the plain model rates highest or next to it
+    llm16 = LLM(str(folder), precision="bfloat16", max_len=128, max_bsz=3, page_size=8)
+    for p, r in zip(prompts, llm16.generate(prompt_token_ids=prompts, temperature=0.0, max_new_tokens=4)):
+        logits = plain.forward(cfg, w64, p)[-1]
+        assert logits[r.token_ids[0]] >= logits.max() - 0.05 * float(logits.std())
+
+
+def test_trace_replay_program(tmp_path):
+    """``bin/trace_run`` as a process: steps in, logits files out, the plain model's values."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    root = Path(__file__).resolve().parent.parent
+    folder = models.make_folder(tmp_path / "m", models.CONFIGS["C"], seed=6)
+    cfg, weights = models.read_folder(folder)
+    requests = {"x": random_tokens(50, cfg["vocab"], 1), "y": random_tokens(90, cfg["vocab"], 2), "z": random_tokens(20, cfg["vocab"], 3)}
+    truth, scale = truth_of(cfg, weights, requests)
+    steps = schedules.mixed(requests, max_live=2)
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, str(root / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32", "--out", str(out),
+         "--max-tokens", str(schedules.max_live_tokens(steps))],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(steps))]
+    for step, rows in zip(steps, schedules.positions_of(steps)):
+        got = torch.from_numpy(np.fromfile(out / f"{step['step']}.f32", dtype="<f4").reshape(len(rows), -1))
+        for row, (rid, pos) in zip(got, rows):
+            assert distance(row, truth[rid][pos], scale) < FP32_TOL
