@@ -2,7 +2,7 @@
 bfloat16 weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
-                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products]
+                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products|taluvik]
 
 Everything runs through the generation loop: the scheduler admits the requests, cuts their prompts
 into portions under its token budget, and plans every decode step; the step function runs it; the
@@ -28,7 +28,8 @@ a read of 4 GiB with 16-byte loads, a device copy, a loop of MFMA instructions o
 library's large matrix product.  ``--workload small-kernels`` times what a norm kernel adds to a
 replayed graph of large products, without a profiler (under rocprofv3 no dispatch is shorter than
 about 4.6 us, an empty kernel included, so a kernel trace overstates the small kernels of a step).
-``--workload attention``: the decode attention and the merge of its splits alone, by batch size, context and
+``--workload taluvik``: prefill and decode of a Taluvik model (chunked attention with sinks, gated delta
+rule, selective scan) beside a Llama model of the same layer sizes.  ``--workload attention``: the decode attention and the merge of its splits alone, by batch size, context and
 split size.  ``--workload products``: a decode layer's four products alone at 1 to 128 rows, the library against
 this package's kernels.  Both as a step runs them: in a replayed graph, caches flushed.
 """
@@ -82,7 +83,8 @@ def parse_args(argv=None):
     p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the headline's)")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products"])
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products", "taluvik"])
+    p.add_argument("--only", default=None, choices=["taluvik", "llama"], help="taluvik: measure one of the two models only")
     p.add_argument("--token-budget", type=int, default=8192, help="tokens a step may hold (the scheduler cuts prompts to it)")
     p.add_argument("--no-reference-workload", action="store_true",
                    help="leave out the reference's benchmark (2,048-token prompts, 256 new tokens at batch 1, 8, 64)")
@@ -289,6 +291,79 @@ def serve_run(args, shape) -> int:
         "seconds": round(sec, 3), "prompt_tokens": prompt_tokens, "generated_tokens": generated,
         "total_tokens_per_s": round((prompt_tokens + generated) / sec, 1),
         "preemptions": loop.scheduler.stats["preemptions"], "prepared_steps": loop.stats["prepared_steps"],
+    }))
+    return 0
+
+
+def taluvik_config(shape: dict, n_layers: int, chunk: int) -> dict:
+    """A Taluvik configuration with the layer sizes of ``shape`` (a Llama configuration): the same
+    width, feed-forward, heads and head size; the delta layers with half as many key heads as heads,
+    the scan layers with twice the width inside, sixteen states and a step-size rank of width / 16;
+    the mixers take turns (scan, attention, delta, scan)."""
+    D, H, G, dh = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    ff = {"kind": "dense", "ff": shape["intermediate_size"]}
+    rs = shape["rope_scaling"]
+    mixers = {
+        "attention": {"heads": H, "kv_heads": G, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "softcap": 30.0, "mask": {"size": chunk},
+                      "rot": {"dims": dh, "base": shape["rope_theta"],
+                              "scaling": {"factor": rs["factor"], "low": rs["low_freq_factor"], "high": rs["high_freq_factor"],
+                                          "original": rs["original_max_position_embeddings"]}}},
+        "delta": {"heads": H, "kv_heads": max(H // 2, 1), "dim": dh, "vdim": dh, "conv": 4},
+        "mamba1": {"inner": 2 * D, "state": 16, "dt_rank": D // 16, "conv": 4},
+    }
+    turn = ["mamba1", "attention", "delta", "mamba1"]
+    return {"architecture": "Taluvik", "vocab": shape["vocab_size"], "width": D, "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-5}, "residual_mult": 1.0,
+            "layers": [{"type": turn[i % 4], "mixer": mixers[turn[i % 4]], "mlp": ff} for i in range(n_layers)]}
+
+
+def taluvik_run(args, shape) -> int:
+    """Prefill and decode of a Taluvik model beside a Llama model of the same layer sizes and number of
+    layers, both with random weights, both through the same engine, scheduler and generation loop:
+    a prompt of ``--prefill-tokens`` in one step (tokens/s), and decode steps of whole batches whose
+    context ends at ``--context`` (ms a step, tokens/s), at ``--batch`` and ``--points``."""
+    import torch
+
+    from torchllms_amd.config import LlamaConfig, TaluvikConfig
+    from torchllms_amd.engine import Engine
+    from torchllms_amd.sampling import Sampler
+
+    n_layers = args.layers or 8
+    batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
+    pages_per_req = -(-max(args.context, args.prefill_tokens) // args.page_size) + 1
+    configs = {
+        "taluvik": TaluvikConfig.from_dict(taluvik_config(shape, n_layers, chunk=8192)),
+        "llama": LlamaConfig.from_dict(dict(shape, num_hidden_layers=n_layers)),
+    }
+    if args.only:
+        configs = {k: v for k, v in configs.items() if k == args.only}
+    new_tokens = 1 + 2 + 3 + args.warmup + args.steps + 1
+    out = {}
+    for name, cfg in configs.items():
+        engine = Engine.from_random(cfg, seed=0, dtype=args.dtype, draw_on_device=True, page_size=args.page_size,
+                                    num_pages=max(batches) * pages_per_req, max_seqs=max(batches), max_model_len=max(args.context, args.prefill_tokens))
+        vocab = engine.vocab_size
+        res = {"weight_bytes": weight_bytes(engine)}
+        sec = prefill_run(engine, args.prefill_tokens, vocab)
+        res["prefill"] = {"tokens": args.prefill_tokens, "ms": round(sec * 1e3, 3), "tokens_per_s": round(args.prefill_tokens / sec, 1)}
+        for b in batches:
+            r = generation_run(engine, Sampler(), b, args.context - new_tokens, new_tokens, vocab, budget=b * args.context,
+                               look_ahead=not args.no_look_ahead, timed_steps=args.steps, warmup=args.warmup)
+            ms = r["timed_s"] / args.steps * 1e3
+            res[f"decode_b{b}"] = {"ms_per_step": round(ms, 4), "tokens_per_s": round(b / ms * 1e3, 1)}
+        out[name] = res
+        del engine
+        torch.cuda.empty_cache()
+    first = next(iter(out.values()))
+    ms = first[f"decode_b{args.batch}"]["ms_per_step"]
+    print(json.dumps({
+        "metric": f"decode tok/s, batch {args.batch}, context {args.context}, Taluvik beside Llama at {SHAPE_NAMES[args.shape]} layer sizes, {n_layers} layers",
+        "value": first[f"decode_b{args.batch}"]["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random-init weights, random token ids",
+        "config": {"model": f"Taluvik and Llama at {SHAPE_NAMES[args.shape]} layer sizes", "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single GPU", "n_layers": n_layers, "page_size": args.page_size},
+        "models": out,
     }))
     return 0
 
@@ -522,6 +597,8 @@ def main(argv=None) -> int:
         return products_run(args, shape)
     if args.workload == "peaks":
         return peaks_run(args)
+    if args.workload == "taluvik":
+        return taluvik_run(args, shape)
     import torch
 
     from torchllms_amd.config import LlamaConfig

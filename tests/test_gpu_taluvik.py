@@ -121,6 +121,7 @@ ALONE = {
                                                  scaling={"factor": 4.0, "low": 1.0, "high": 4.0, "original": 16})),
     "delta": models.layer("delta", {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 40, "conv": 4}),
     "delta_wide": models.layer("delta", {"heads": 1, "kv_heads": 1, "dim": 256, "vdim": 64, "conv": 2}),
+    "delta_odd": models.layer("delta", {"heads": 3, "kv_heads": 1, "dim": 18, "vdim": 70, "conv": 3}),
     "mamba1": models.layer("mamba1", {"inner": 72, "state": 24, "dt_rank": 6, "conv": 3}),
     "mamba1_many_states": models.layer("mamba1", {"inner": 40, "state": 100, "dt_rank": 8, "conv": 6}),
     "feed_forward": models.layer("mamba1", {"inner": 8, "state": 1, "dt_rank": 1, "conv": 1}, ff=136),
@@ -283,6 +284,40 @@ def test_long_decoding_from_recorded_steps(tmp_path, dtype):
             worst = max(worst, distance(row, truth[rid][heads[rid] + i], scale))
     assert any(g.replays > 100 for g in engine.graphs.graphs.values())
     assert worst < tol, worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompts_beside_short_ones(tmp_path, dtype):
+    """Prompts of several hundred tokens in one step, beside a short portion and a single token of
+    other requests: in bfloat16 the selective scan cuts long rows into segments that run side by side
+    (the last one shorter), and the delta rule's tiles and the attention's chunks end inside them."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    folder = models.make_folder(tmp_path / "m", models.CONFIGS["A"], seed=12)
+    cfg, weights = models.read_folder(folder)
+    requests = {"long": random_tokens(700, cfg["vocab"], 1), "mid": random_tokens(333, cfg["vocab"], 2),
+                "short": random_tokens(40, cfg["vocab"], 3), "one": random_tokens(9, cfg["vocab"], 4)}
+    truth, scale = truth_of(cfg, weights, requests)
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=160, max_seqs=4)
+    for rid in requests:
+        engine.admit(rid)
+    engine.step([StepEntry("short", requests["short"][:31], []), StepEntry("one", requests["one"][:8], [])])
+    wanted = {"long": [0, 63, 64, 255, 256, 639, 640, 699], "mid": [0, 100, 320, 332], "short": list(range(9)), "one": [0]}
+    entries = [StepEntry("long", requests["long"], wanted["long"]), StepEntry("one", requests["one"][8:], [0]),
+               StepEntry("mid", requests["mid"], wanted["mid"]), StepEntry("short", requests["short"][31:], wanted["short"])]
+    logits = engine.step(entries).cpu()
+    tol = FP32_TOL if dtype == "float32" else BF16_TOL
+    at = 0
+    for e, base in zip(entries, (0, 8, 0, 31)):
+        for w in e.want:
+            d = distance(logits[at], truth[e.rid][base + w], scale)
+            assert d < tol, f"{e.rid} at {base + w}: distance {d}"
+            at += 1
+    # and the states that the long rows left behind carry on
+    more = engine.step([StepEntry("long", [5], [0]), StepEntry("mid", [7], [0])]).cpu()
+    w64 = {k: v.double() for k, v in weights.items()}
+    for row, (rid, tok) in zip(more, (("long", 5), ("mid", 7))):
+        assert distance(row, plain.forward(cfg, w64, requests[rid] + [tok])[-1], scale) < tol
 
 
 def test_greedy_generation_through_the_entry_point(tmp_path):

@@ -97,14 +97,32 @@ int layernorm_launch(const void* x, const void* d0, const void* d1, float mult, 
 
 // ----------------------------------------------------------------------------- gated activation
 // gate_up: [n, 2F] = gate | up.  out[n, F] = T(act(float(gate)) * float(up)); act 1: gelu in its tanh form.
-template <typename T>
+// A thread takes V consecutive columns of one row (V elements = 16 bytes when the row allows it).
+template <typename T, int V>
 __global__ void gelu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int n, int inter) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= inter) return;
+  const int c0 = (blockIdx.x * blockDim.x + threadIdx.x) * V;
+  if (c0 >= inter) return;
+  struct alignas(sizeof(T) * V) Vec { T e[V]; };
   for (int r = blockIdx.y; r < n; r += gridDim.y) {
-    const T* gp = gate_up + (size_t)r * 2 * inter + c;
-    out[(size_t)r * inter + c] = from_f32<T>(gelu_tanh_f(to_f32(gp[0])) * to_f32(gp[inter]));
+    const T* gp = gate_up + (size_t)r * 2 * inter + c0;
+    const Vec g = *reinterpret_cast<const Vec*>(gp);
+    const Vec u = *reinterpret_cast<const Vec*>(gp + inter);
+    Vec o;
+#pragma unroll
+    for (int i = 0; i < V; ++i) o.e[i] = from_f32<T>(gelu_tanh_f(to_f32(g.e[i])) * to_f32(u.e[i]));
+    *reinterpret_cast<Vec*>(out + (size_t)r * inter + c0) = o;
   }
+}
+
+template <typename T>
+int gelu_mul_launch(const T* gate_up, T* out, int n, int inter, hipStream_t stream) {
+  constexpr int kVec = 16 / sizeof(T);
+  const bool wide = inter % kVec == 0 && ((uintptr_t)gate_up % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  const int per_block = 256 * (wide ? kVec : 1);
+  const dim3 grid((inter + per_block - 1) / per_block, n < 65535 ? n : 65535);
+  if (wide) gelu_mul_kernel<T, kVec><<<grid, 256, 0, stream>>>(gate_up, out, n, inter);
+  else gelu_mul_kernel<T, 1><<<grid, 256, 0, stream>>>(gate_up, out, n, inter);
+  return tl_check_launch("gelu_mul");
 }
 
 // ----------------------------------------------------------------------------- rotation, unit norm, cache write
@@ -238,31 +256,39 @@ conv_history_kernel(const T* __restrict__ x, int x_stride, float* __restrict__ s
 constexpr int kScanThreads = 128;
 constexpr int kScanTile = 8;
 
-template <typename T, typename DT, int NB>
+// MODE 0: a block walks all tokens of its request, from the request's state to the request's state.
+// For long prompts the walk is cut into segments of tokens that run side by side (``segs``: first and
+// last token of every segment): MODE 1 walks a segment from a zero state, emits nothing and leaves the
+// state it ends with and the sum of its step sizes (the decay of state n over the segment is
+// exp(A[c][n] * that sum)); a carry kernel then goes over each request's segments in order and puts the
+// state that enters each in its place; MODE 2 walks the segment again from there and emits.
+template <typename T, typename DT, int NB, int MODE>
 __global__ void __launch_bounds__(kScanThreads)
 selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, const T* __restrict__ bc, int bc_stride,
                       int b_off, int c_off, const T* __restrict__ z, int z_stride, const float* __restrict__ dt_bias,
                       const float* __restrict__ A, const float* __restrict__ D, float* __restrict__ state,
                       long long state_stride, const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ slot_ids,
-                      T* __restrict__ out, int inner, int N, int lpc) {
+                      T* __restrict__ out, int inner, int N, int lpc, const int32_t* __restrict__ segs,
+                      float* __restrict__ seg_dt) {
   extern __shared__ float bc_lds[];  // [kScanTile][2 * N]
-  const int row = blockIdx.y;
-  const int start = qo_indptr[row], end = qo_indptr[row + 1];
+  const int row = blockIdx.y;  // (MODE 1, 2: the segment)
+  const int start = MODE == 0 ? qo_indptr[row] : segs[2 * row], end = MODE == 0 ? qo_indptr[row + 1] : segs[2 * row + 1];
   const int per_block = kScanThreads / lpc;
   const int c_raw = blockIdx.x * per_block + threadIdx.x / lpc;
   const int part = threadIdx.x % lpc;
   const bool live = c_raw < inner;
   const int c = live ? c_raw : inner - 1;
   const int n0 = part * NB;
-  float* st = state + (long long)slot_ids[row] * state_stride + (size_t)c * N;
+  float* st = state + (MODE == 0 ? (long long)slot_ids[row] : (long long)row) * state_stride + (size_t)c * N;
   float s[NB], a[NB];
 #pragma unroll
   for (int n = 0; n < NB; ++n) {
     const bool in = n0 + n < N;
-    s[n] = in ? st[n0 + n] : 0.f;
+    s[n] = in && MODE != 1 ? st[n0 + n] : 0.f;
     a[n] = in ? A[(size_t)c * N + n0 + n] : 0.f;
   }
   const float bias = dt_bias[c], dd = D[c];
+  float dt_sum = 0.f;
   for (int t0 = start; t0 < end; t0 += kScanTile) {
     const int nt = min(kScanTile, end - t0);
     __syncthreads();  // everybody has finished with the tile before
@@ -276,8 +302,9 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
       const size_t t = (size_t)(t0 + tt);
       const float xv = to_f32(x[t * inner + c]);
       const float dt = softplus_f(to_f32(dt_pre[t * inner + c]) + bias);
-      const float zv = to_f32(z[t * z_stride + c]);
+      const float zv = MODE == 1 ? 0.f : to_f32(z[t * z_stride + c]);
       const float dx = dt * xv;
+      dt_sum += dt;
       const float* Bt = bc_lds + tt * 2 * N + n0;
       const float* Ct = Bt + N;
       float y = 0.f;
@@ -288,16 +315,43 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
           y = fmaf(s[n], Ct[n], y);
         }
       }
-      y = group_sum(y, lpc);
-      y = fmaf(dd, xv, y);
-      if (live && part == 0) out[t * inner + c] = from_f32<T>(y * silu_f(zv));
+      if (MODE != 1) {
+        y = group_sum(y, lpc);
+        y = fmaf(dd, xv, y);
+        if (live && part == 0) out[t * inner + c] = from_f32<T>(y * silu_f(zv));
+      }
     }
   }
-  if (live) {
+  if (live && MODE != 2) {
 #pragma unroll
     for (int n = 0; n < NB; ++n)
       if (n0 + n < N) st[n0 + n] = s[n];
+    if (MODE == 1 && part == 0) seg_dt[(size_t)row * inner + c] = dt_sum;
   }
+}
+
+// The carry between the segments of a request: element (c, n) of the state goes through the request's
+// segments in order; ws[seg] holds the state a segment ends with when it starts from zero and receives
+// the state that enters it.  The request's state row takes what the last segment leaves.
+__global__ void __launch_bounds__(256)
+scan_carry_kernel(float* __restrict__ ws, const float* __restrict__ seg_dt, const float* __restrict__ A,
+                  float* __restrict__ state, long long state_stride, const int32_t* __restrict__ row_seg,
+                  const int32_t* __restrict__ slot_ids, int inner, int N) {
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t per = (size_t)inner * N;
+  if (idx >= per) return;
+  const int row = blockIdx.y;
+  const int c = (int)(idx / N);
+  float* st = state + (long long)slot_ids[row] * state_stride + idx;
+  float s = *st;
+  const float a = A[idx];
+  for (int seg = row_seg[row]; seg < row_seg[row + 1]; ++seg) {
+    float* w = ws + (size_t)seg * per + idx;
+    const float local = *w;
+    *w = s;
+    s = fmaf(expf(a * seg_dt[(size_t)seg * inner + c]), s, local);
+  }
+  *st = s;
 }
 
 // ----------------------------------------------------------------------------- gated delta rule
@@ -306,112 +360,200 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
 //   k^ = k / sqrt(sum k^2 + 1e-6);  q^ = q / sqrt(sum q^2 + 1e-6) * dk^-1/2
 //   beta = sigmoid(b);  decay = exp(-exp(A_log[h]) * softplus(a + dt_bias[h]))
 //   S <- decay * S;  u = beta * (v - S^T k^);  S <- S + k^ u^T;  o = S^T q^
-//   out[t, h, :] = T(o / sqrt(mean(o^2) + eps) * norm_w * silu(gate[t, h, :]))
+// and, in a second kernel, out[t, h, :] = T(o / sqrt(mean(o^2) + eps) * norm_w * silu(gate[t, h, :])).
 // qkv: the convolved and activated q | k | v channels, [n_tokens, qkv_stride]; proj: the layer's input
 // projection, of which gate (H * dv columns from gate_off), b and a (H columns each) are read.
-// A block is one (request, head); lpc neighbouring lanes share column j, each holding RB rows of it.
-constexpr int kDeltaTile = 8;
+//
+// The columns of S do not depend on each other, so a block takes kDeltaCols columns of one (request,
+// head): a prompt of one request fills the GPU with heads * dv / kDeltaCols blocks.  lpc neighbouring
+// lanes share a column, each holding 16 rows of it in registers.  The tokens come in tiles of kDeltaTile:
+// the raw keys, queries and values of the next tile travel from memory into registers while the current
+// tile is worked on; in LDS the keys and queries are made unit vectors once per tile; then the tile's
+// tokens follow each other without a barrier (sums over a column's lanes by lane-to-lane moves).
+constexpr int kDeltaTile = 16;
+constexpr int kDeltaCols = 32;
+constexpr int kDeltaRows = 16;  // rows of a column that a lane holds
 
-template <typename T, int RB>
-__global__ void __launch_bounds__(1024)
-gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int gate_off,
-                   int b_off, int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
-                   const float* __restrict__ norm_w, float eps, float* __restrict__ state, long long state_stride,
-                   const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ slot_ids, T* __restrict__ out,
-                   int H, int G, int dk, int dv, int lpc) {
-  extern __shared__ float lds[];
-  // per token of the tile: k^ [dk], q^ [dk], v [dv], o [dv], then beta and decay
+// Sum over groups of `width` neighbouring lanes (1, 2, 4, 8 or 16) by data-parallel moves inside a row
+// of 16 lanes: every lane of a group gets the same bits.
+__device__ __forceinline__ float dpp_xor1(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float dpp_xor2(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float dpp_half_mirror(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float dpp_mirror(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float row_group_sum(float v, int width) {
+  if (width >= 2) v += dpp_xor1(v);
+  if (width >= 4) v += dpp_xor2(v);
+  if (width >= 8) v += dpp_half_mirror(v);
+  if (width >= 16) v += dpp_mirror(v);
+  return v;
+}
+
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(512)
+gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int b_off,
+                   int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+                   float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
+                   const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int dk, int dv, int lpc,
+                   int col_groups) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // per token of the tile: k [dk], q [dk] (raw, then unit), v [kDeltaCols], o [kDeltaCols]; then beta, decay, 1/|k|, scale/|q|
   float* k_l = lds;
   float* q_l = k_l + kDeltaTile * dk;
   float* v_l = q_l + kDeltaTile * dk;
-  float* o_l = v_l + kDeltaTile * dv;
-  float* bd_l = o_l + kDeltaTile * dv;  // [kDeltaTile][2]
-  const int row = blockIdx.y, h = blockIdx.x;
+  float* o_l = v_l + kDeltaTile * kDeltaCols;
+  float* sc_l = o_l + kDeltaTile * kDeltaCols;  // [kDeltaTile][4]
+  const int row = blockIdx.y;
+  const int h = blockIdx.x / col_groups, cg = blockIdx.x % col_groups;
   const int g = h / (H / G);
   const int start = qo_indptr[row], end = qo_indptr[row + 1];
-  const int n_threads = blockDim.x, n_waves = n_threads / kWave;
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int j_raw = threadIdx.x / lpc, part = threadIdx.x % lpc;
-  const bool live = j_raw < dv;
-  const int j = live ? j_raw : dv - 1;
-  const int i0 = part * RB;
+  const int n_threads = blockDim.x;
+  const int j_loc = threadIdx.x / lpc, part = threadIdx.x % lpc;
+  const int j_raw = cg * kDeltaCols + j_loc;
+  const bool live = j_loc < kDeltaCols && j_raw < dv;
+  const int j = j_raw < dv ? j_raw : dv - 1;
+  const int i0 = part * kDeltaRows;
   float* st = state + (long long)slot_ids[row] * state_stride + ((size_t)h * dv + j) * dk;
-  float S[RB];
+  float S[kDeltaRows];
 #pragma unroll
-  for (int r = 0; r < RB; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
+  for (int r = 0; r < kDeltaRows; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
   const float neg_rate = -expf(A_log[h]), bias = dt_bias[h];
   const float q_scale = 1.0f / sqrtf((float)dk);
-  const int q_col = g * dk, k_col = G * dk + g * dk, v_col = 2 * G * dk + h * dv;
+  const int q_col = g * dk, k_col = G * dk + g * dk, v_col = 2 * G * dk + h * dv + cg * kDeltaCols;
+  const int v_cols = min(kDeltaCols, dv - cg * kDeltaCols);
+
+  // what a thread fetches of a tile: element e of the tile's keys and queries (e = tt * 2 dk + d, d < dk a
+  // key's channel, else a query's) for e = tid, tid + threads, ...; likewise of the values
+  constexpr int kPreKQ = 16, kPreV = 8;
+  T pre_kq[kPreKQ], pre_v[kPreV];
+  auto fetch = [&](int t0) {
+    const int nt = min(kDeltaTile, end - t0);
+#pragma unroll
+    for (int u = 0; u < kPreKQ; ++u) {
+      const int e = threadIdx.x + u * n_threads;
+      const int tt = e / (2 * dk), d = e % (2 * dk);
+      if (tt < nt) pre_kq[u] = qkv[(size_t)(t0 + tt) * qkv_stride + (d < dk ? k_col + d : q_col + d - dk)];
+    }
+#pragma unroll
+    for (int u = 0; u < kPreV; ++u) {
+      const int e = threadIdx.x + u * n_threads;
+      const int tt = e / kDeltaCols, d = e % kDeltaCols;
+      if (tt < nt && d < v_cols) pre_v[u] = qkv[(size_t)(t0 + tt) * qkv_stride + v_col + d];
+    }
+  };
+  if (start < end) fetch(start);
   for (int t0 = start; t0 < end; t0 += kDeltaTile) {
     const int nt = min(kDeltaTile, end - t0);
-    __syncthreads();  // the tile before has been written out
-    // unit keys and queries: one wave per (token, which)
-    for (int item = wave; item < 2 * nt; item += n_waves) {
-      const int tt = item / 2, which = item % 2;  // 0: k, 1: q
-      const T* src = qkv + (size_t)(t0 + tt) * qkv_stride + (which ? q_col : k_col);
-      float ss = 0.f;
-      for (int d = lane; d < dk; d += kWave) {
-        const float v = to_f32(src[d]);
-        ss += v * v;
-      }
-      ss = wave_sum(ss);
-      const float inv = (which ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
-      float* dst = (which ? q_l : k_l) + tt * dk;
-      for (int d = lane; d < dk; d += kWave) dst[d] = to_f32(src[d]) * inv;
+    __syncthreads();  // the tile before has been read to its end
+#pragma unroll
+    for (int u = 0; u < kPreKQ; ++u) {
+      const int e = threadIdx.x + u * n_threads;
+      const int tt = e / (2 * dk), d = e % (2 * dk);
+      if (tt < nt) (d < dk ? k_l[tt * dk + d] : q_l[tt * dk + d - dk]) = to_f32(pre_kq[u]);
     }
-    for (int idx = threadIdx.x; idx < nt * dv; idx += n_threads) {
-      const int tt = idx / dv, d = idx % dv;
-      v_l[idx] = to_f32(qkv[(size_t)(t0 + tt) * qkv_stride + v_col + d]);
+#pragma unroll
+    for (int u = 0; u < kPreV; ++u) {
+      const int e = threadIdx.x + u * n_threads;
+      const int tt = e / kDeltaCols, d = e % kDeltaCols;
+      if (tt < nt && d < v_cols) v_l[tt * kDeltaCols + d] = to_f32(pre_v[u]);
     }
     if (threadIdx.x < nt) {
       const T* pr = proj + (size_t)(t0 + threadIdx.x) * proj_stride;
-      bd_l[2 * threadIdx.x] = sigmoid_f(to_f32(pr[b_off + h]));
-      bd_l[2 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pr[a_off + h]) + bias));
+      sc_l[4 * threadIdx.x] = sigmoid_f(to_f32(pr[b_off + h]));
+      sc_l[4 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pr[a_off + h]) + bias));
+    }
+    if (t0 + kDeltaTile < end) fetch(t0 + kDeltaTile);  // on its way while this tile is worked on
+    __syncthreads();
+    // the norms: 2 nt vectors, each summed by one thread in ascending order of its channels
+    if (threadIdx.x < 2 * nt) {
+      const int tt = threadIdx.x / 2, which = threadIdx.x % 2;
+      const float* src = (which ? q_l : k_l) + tt * dk;
+      float ss = 0.f;
+      for (int d = 0; d < dk; ++d) ss = fmaf(src[d], src[d], ss);
+      sc_l[4 * tt + 2 + which] = (which ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nt * 2 * dk; e += n_threads) {
+      const int tt = e / (2 * dk), d = e % (2 * dk);
+      if (d < dk) k_l[tt * dk + d] *= sc_l[4 * tt + 2];
+      else q_l[tt * dk + d - dk] *= sc_l[4 * tt + 3];
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const float beta = bd_l[2 * tt], decay = bd_l[2 * tt + 1];
+      const float beta = sc_l[4 * tt], decay = sc_l[4 * tt + 1];
       const float* kt = k_l + tt * dk + i0;
       const float* qt = q_l + tt * dk + i0;
-      float kv = 0.f;
+      float kk[kDeltaRows], qq[kDeltaRows];
+      if (VEC) {  // dk is a multiple of 4: four channels a read
 #pragma unroll
-      for (int r = 0; r < RB; ++r) {
-        if (i0 + r < dk) {
-          S[r] = decay * S[r];
-          kv = fmaf(S[r], kt[r], kv);
+        for (int r = 0; r < kDeltaRows; r += 4) {
+          const bool in = i0 + r < dk;
+          const float4 k4 = in ? *reinterpret_cast<const float4*>(kt + r) : float4{0.f, 0.f, 0.f, 0.f};
+          const float4 q4 = in ? *reinterpret_cast<const float4*>(qt + r) : float4{0.f, 0.f, 0.f, 0.f};
+          kk[r] = k4.x; kk[r + 1] = k4.y; kk[r + 2] = k4.z; kk[r + 3] = k4.w;
+          qq[r] = q4.x; qq[r + 1] = q4.y; qq[r + 2] = q4.z; qq[r + 3] = q4.w;
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < kDeltaRows; ++r) {
+          kk[r] = i0 + r < dk ? kt[r] : 0.f;
+          qq[r] = i0 + r < dk ? qt[r] : 0.f;
         }
       }
-      kv = group_sum(kv, lpc);
-      const float u = beta * (v_l[tt * dv + j] - kv);
-      float o = 0.f;
+      float kv[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int r = 0; r < RB; ++r) {
-        if (i0 + r < dk) {
-          S[r] = fmaf(kt[r], u, S[r]);
-          o = fmaf(S[r], qt[r], o);
-        }
+      for (int r = 0; r < kDeltaRows; ++r) {
+        S[r] = decay * S[r];
+        kv[r % 4] = fmaf(S[r], kk[r], kv[r % 4]);
       }
-      o = group_sum(o, lpc);
-      if (live && part == 0) o_l[tt * dv + j] = o;
+      const float kv_all = row_group_sum((kv[0] + kv[1]) + (kv[2] + kv[3]), lpc);
+      const float u = beta * (v_l[tt * kDeltaCols + (j_loc < kDeltaCols ? j_loc : 0)] - kv_all);
+      float o[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < kDeltaRows; ++r) {
+        S[r] = fmaf(kk[r], u, S[r]);
+        o[r % 4] = fmaf(S[r], qq[r], o[r % 4]);
+      }
+      const float o_all = row_group_sum((o[0] + o[1]) + (o[2] + o[3]), lpc);
+      if (live && part == 0) o_l[tt * kDeltaCols + j_loc] = o_all;
     }
     __syncthreads();
-    // per-head RMS norm of the outputs, the norm's weight and the gate: one wave per token
-    for (int tt = wave; tt < nt; tt += n_waves) {
-      float ss = 0.f;
-      for (int d = lane; d < dv; d += kWave) ss += o_l[tt * dv + d] * o_l[tt * dv + d];
-      ss = wave_sum(ss);
-      const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
-      const T* gp = proj + (size_t)(t0 + tt) * proj_stride + gate_off + (size_t)h * dv;
-      T* op = out + ((size_t)(t0 + tt) * H + h) * dv;
-      for (int d = lane; d < dv; d += kWave)
-        op[d] = from_f32<T>(o_l[tt * dv + d] * inv * norm_w[d] * silu_f(to_f32(gp[d])));
+    for (int e = threadIdx.x; e < nt * v_cols; e += n_threads) {
+      const int tt = e / v_cols, d = e % v_cols;
+      o_raw[((size_t)(t0 + tt) * H + h) * dv + cg * kDeltaCols + d] = o_l[tt * kDeltaCols + d];
     }
   }
   if (live) {
 #pragma unroll
-    for (int r = 0; r < RB; ++r)
+    for (int r = 0; r < kDeltaRows; ++r)
       if (i0 + r < dk) st[i0 + r] = S[r];
   }
+}
+
+// out[t, h, :] = T(o / sqrt(mean(o^2) + eps) * norm_w * silu(gate[t, h, :])): one wave a (token, head).
+template <typename T>
+__global__ void __launch_bounds__(kHeadWaves* kWave)
+delta_output_kernel(const float* __restrict__ o_raw, const T* __restrict__ proj, int proj_stride, int gate_off,
+                    const float* __restrict__ norm_w, float eps, T* __restrict__ out, int H, int dv) {
+  const int t = blockIdx.x;
+  const int h = blockIdx.y * kHeadWaves + threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave;
+  if (h >= H) return;
+  const float* o = o_raw + ((size_t)t * H + h) * dv;
+  float ss = 0.f;
+  for (int d = lane; d < dv; d += kWave) ss = fmaf(o[d], o[d], ss);
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+  const T* gp = proj + (size_t)t * proj_stride + gate_off + (size_t)h * dv;
+  T* op = out + ((size_t)t * H + h) * dv;
+  for (int d = lane; d < dv; d += kWave) op[d] = from_f32<T>(o[d] * inv * norm_w[d] * silu_f(to_f32(gp[d])));
 }
 
 }  // namespace
@@ -451,14 +593,9 @@ TL_EXPORT int tl_layernorm(const void* x, const void* d0, const void* d1, float 
 TL_EXPORT int tl_gelu_mul(const void* gate_up, void* out, int n, int inter, int dtype, hipStream_t stream) {
   TL_REQUIRE(n >= 0 && inter > 0, "gelu_mul: bad sizes n=%d inter=%d", n, inter);
   if (n == 0) return TL_OK;
-  const dim3 grid((inter + 255) / 256, n < 65535 ? n : 65535);
-  if (dtype == TL_F32)
-    gelu_mul_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up, (float*)out, n, inter);
-  else if (dtype == TL_BF16)
-    gelu_mul_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, n, inter);
-  else
-    return tl_fail(TL_ERR_ARG, "gelu_mul: unknown dtype %d", dtype);
-  return tl_check_launch("gelu_mul");
+  if (dtype == TL_F32) return gelu_mul_launch((const float*)gate_up, (float*)out, n, inter, stream);
+  if (dtype == TL_BF16) return gelu_mul_launch((const bf16_t*)gate_up, (bf16_t*)out, n, inter, stream);
+  return tl_fail(TL_ERR_ARG, "gelu_mul: unknown dtype %d", dtype);
 }
 
 TL_EXPORT int tl_rope_norm_kv_write(void* qkv, int n_tokens, int n_q, int n_kv, int dk, int dv, const float* cos_sin, int rot,
@@ -523,92 +660,111 @@ namespace {
 template <typename T, typename DT>
 int scan_launch(const void* x, const void* dt_pre, const void* bc, int bc_stride, int b_off, int c_off, const void* z,
                 int z_stride, const float* dt_bias, const float* A, const float* D, float* state, long long state_stride,
-                const int32_t* qo_indptr, const int32_t* slot_ids, void* out, int n_seqs, int inner, int N, hipStream_t stream) {
+                const int32_t* qo_indptr, const int32_t* slot_ids, void* out, int n_seqs, int inner, int N,
+                const int32_t* segs, const int32_t* row_seg, int n_segs, float* ws, float* seg_dt, hipStream_t stream) {
   // states a lane holds and lanes a channel: up to 32 states one lane, then 2, 4, 8 lanes of 32
   int nb = N <= 8 ? 8 : N <= 16 ? 16 : 32;
   int lpc = 1;
   while (nb * lpc < N) lpc *= 2;
   const int per_block = kScanThreads / lpc;
-  const dim3 grid((inner + per_block - 1) / per_block, n_seqs);
+  const int cblocks = (inner + per_block - 1) / per_block;
   const size_t lds = (size_t)kScanTile * 2 * N * sizeof(float);
-#define TL_SCAN(NB)                                                                                                     \
-  selective_scan_kernel<T, DT, NB><<<grid, kScanThreads, lds, stream>>>(                                                \
-      (const T*)x, (const DT*)dt_pre, (const T*)bc, bc_stride, b_off, c_off, (const T*)z, z_stride, dt_bias, A, D, state, \
-      state_stride, qo_indptr, slot_ids, (T*)out, inner, N, lpc)
-  if (nb == 8) TL_SCAN(8);
-  else if (nb == 16) TL_SCAN(16);
-  else TL_SCAN(32);
+#define TL_SCAN(NB, MODE, ROWS, STATE, STRIDE)                                                                          \
+  selective_scan_kernel<T, DT, NB, MODE><<<dim3(cblocks, ROWS), kScanThreads, lds, stream>>>(                           \
+      (const T*)x, (const DT*)dt_pre, (const T*)bc, bc_stride, b_off, c_off, (const T*)z, z_stride, dt_bias, A, D, STATE, \
+      STRIDE, qo_indptr, slot_ids, (T*)out, inner, N, lpc, segs, seg_dt)
+#define TL_SCAN_NB(MODE, ROWS, STATE, STRIDE)               \
+  do {                                                      \
+    if (nb == 8) TL_SCAN(8, MODE, ROWS, STATE, STRIDE);     \
+    else if (nb == 16) TL_SCAN(16, MODE, ROWS, STATE, STRIDE); \
+    else TL_SCAN(32, MODE, ROWS, STATE, STRIDE);            \
+  } while (0)
+  if (segs == nullptr) {
+    TL_SCAN_NB(0, n_seqs, state, state_stride);
+    return tl_check_launch("selective_scan");
+  }
+  const long long per = (long long)inner * N;
+  TL_SCAN_NB(1, n_segs, ws, per);
+  int rc = tl_check_launch("selective_scan (segments)");
+  if (rc != TL_OK) return rc;
+  scan_carry_kernel<<<dim3((unsigned)((per + 255) / 256), n_seqs), 256, 0, stream>>>(ws, seg_dt, A, state, state_stride, row_seg,
+                                                                                 slot_ids, inner, N);
+  rc = tl_check_launch("selective_scan (carry)");
+  if (rc != TL_OK) return rc;
+  TL_SCAN_NB(2, n_segs, ws, per);
+#undef TL_SCAN_NB
 #undef TL_SCAN
-  return tl_check_launch("selective_scan");
+  return tl_check_launch("selective_scan (emit)");
 }
 }  // namespace
 
 // x, out: [n_tokens, inner] of dtype; dt_pre: [n_tokens, inner] of dt_dtype (32-bit, or dtype); bc and z: see the
-// kernel; state: the requests' rows, S[c][n] at state + slot * state_stride + c * N + n.
+// kernel; state: the requests' rows, S[c][n] at state + slot * state_stride + c * N + n.  With segs (first and last
+// token of n_segs segments, every request's in order) and row_seg (n_seqs + 1: the first segment of every request)
+// the segments run side by side; ws: n_segs * inner * N floats, seg_dt: n_segs * inner floats.
 TL_EXPORT int tl_selective_scan(const void* x, const void* dt_pre, int dt_dtype, const void* bc, int bc_stride, int b_off,
                                 int c_off, const void* z, int z_stride, const float* dt_bias, const float* A, const float* D,
                                 float* state, long long state_stride, const int32_t* qo_indptr, const int32_t* slot_ids,
-                                void* out, int n_seqs, int inner, int N, int dtype, hipStream_t stream) {
+                                void* out, int n_seqs, int inner, int N, int dtype, const int32_t* segs,
+                                const int32_t* row_seg, int n_segs, float* ws, float* seg_dt, hipStream_t stream) {
   TL_REQUIRE(n_seqs >= 0 && inner > 0 && N > 0, "selective_scan: bad sizes");
   TL_REQUIRE(N <= 256, "selective_scan: %d states a channel, at most 256", N);
-  TL_REQUIRE(n_seqs <= 65535, "selective_scan: at most 65535 requests a step");
+  TL_REQUIRE(n_seqs <= 65535 && n_segs <= 65535, "selective_scan: at most 65535 requests and segments a step");
+  TL_REQUIRE(segs == nullptr || (row_seg != nullptr && ws != nullptr && seg_dt != nullptr && n_segs > 0),
+             "selective_scan: segments without their workspace");
   if (n_seqs == 0) return TL_OK;
-  if (dtype == TL_F32 && dt_dtype == TL_F32)
-    return scan_launch<float, float>(x, dt_pre, bc, bc_stride, b_off, c_off, z, z_stride, dt_bias, A, D, state, state_stride,
-                                     qo_indptr, slot_ids, out, n_seqs, inner, N, stream);
-  if (dtype == TL_BF16 && dt_dtype == TL_F32)
-    return scan_launch<bf16_t, float>(x, dt_pre, bc, bc_stride, b_off, c_off, z, z_stride, dt_bias, A, D, state, state_stride,
-                                      qo_indptr, slot_ids, out, n_seqs, inner, N, stream);
-  if (dtype == TL_BF16 && dt_dtype == TL_BF16)
-    return scan_launch<bf16_t, bf16_t>(x, dt_pre, bc, bc_stride, b_off, c_off, z, z_stride, dt_bias, A, D, state, state_stride,
-                                       qo_indptr, slot_ids, out, n_seqs, inner, N, stream);
+#define TL_SCAN_ARGS x, dt_pre, bc, bc_stride, b_off, c_off, z, z_stride, dt_bias, A, D, state, state_stride, qo_indptr, slot_ids, \
+                     out, n_seqs, inner, N, segs, row_seg, n_segs, ws, seg_dt, stream
+  if (dtype == TL_F32 && dt_dtype == TL_F32) return scan_launch<float, float>(TL_SCAN_ARGS);
+  if (dtype == TL_BF16 && dt_dtype == TL_F32) return scan_launch<bf16_t, float>(TL_SCAN_ARGS);
+  if (dtype == TL_BF16 && dt_dtype == TL_BF16) return scan_launch<bf16_t, bf16_t>(TL_SCAN_ARGS);
+#undef TL_SCAN_ARGS
   return tl_fail(TL_ERR_ARG, "selective_scan: dtype %d with step sizes of dtype %d", dtype, dt_dtype);
 }
 
-// qkv, proj, out as the kernel describes; state: S^T of head h at state + slot * state_stride + h * dv * dk.
+// qkv, proj, out as the kernels describe; state: S^T of head h at state + slot * state_stride + h * dv * dk;
+// o_raw: workspace of n_tokens * H * dv floats.
 TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, int proj_stride, int gate_off, int b_off,
                              int a_off, const float* A_log, const float* dt_bias, const float* norm_w, float eps, float* state,
-                             long long state_stride, const int32_t* qo_indptr, const int32_t* slot_ids, void* out, int n_seqs,
-                             int H, int G, int dk, int dv, int dtype, hipStream_t stream) {
-  TL_REQUIRE(n_seqs >= 0 && H > 0 && G > 0 && dk > 0 && dv > 0, "gated_delta: bad sizes");
+                             long long state_stride, const int32_t* qo_indptr, const int32_t* slot_ids, void* out, int n_tokens,
+                             int n_seqs, int H, int G, int dk, int dv, float* o_raw, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && H > 0 && G > 0 && dk > 0 && dv > 0, "gated_delta: bad sizes");
   TL_REQUIRE(H % G == 0, "gated_delta: %d heads are not a multiple of %d key heads", H, G);
-  TL_REQUIRE(dk <= 1024 && dv <= 1024, "gated_delta: head sizes %d and %d, at most 1024", dk, dv);
-  TL_REQUIRE(n_seqs <= 65535, "gated_delta: at most 65535 requests a step");
-  if (n_seqs == 0) return TL_OK;
-  // rows of a column that a lane holds (16, 32 or 64) and lanes a column, so that a block has at most 1024 threads
-  int rb = 16, lpc = 1;
-  for (;;) {
-    lpc = 1;
-    while (rb * lpc < dk) lpc *= 2;
-    if (lpc <= kWave && (size_t)dv * lpc <= 1024) break;
-    if (rb == 64) return tl_fail(TL_ERR_UNSUPPORTED, "gated_delta: heads of %d by %d do not fit a block", dk, dv);
-    rb *= 2;
+  if (dk > 256) return tl_fail(TL_ERR_UNSUPPORTED, "gated_delta: keys of %d channels, at most 256", dk);
+  TL_REQUIRE(n_seqs <= 65535 && n_tokens <= 0x7fffffff / 4, "gated_delta: too many requests or tokens a step");
+  TL_REQUIRE(o_raw != nullptr, "gated_delta: no workspace");
+  if (n_seqs == 0 || n_tokens == 0) return TL_OK;
+  if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "gated_delta: unknown dtype %d", dtype);
+  int lpc = 1;
+  while (kDeltaRows * lpc < dk) lpc *= 2;  // at most 16: a column's lanes lie in one row of 16 lanes
+  const int threads = (kDeltaCols * lpc + kWave - 1) / kWave * kWave;
+  const int col_groups = (dv + kDeltaCols - 1) / kDeltaCols;
+  const size_t lds = ((size_t)kDeltaTile * (2 * dk + 2 * kDeltaCols + 4)) * sizeof(float);
+  const dim3 grid(H * col_groups, n_seqs);
+#define TL_DELTA(T, VEC)                                                                                               \
+  gated_delta_kernel<T, VEC><<<grid, threads, lds, stream>>>((const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, \
+                                                             a_off, A_log, dt_bias, state, state_stride, qo_indptr, slot_ids, \
+                                                             o_raw, H, G, dk, dv, lpc, col_groups)
+  if (dtype == TL_F32) {
+    if (dk % 4 == 0) TL_DELTA(float, true);
+    else TL_DELTA(float, false);
+  } else {
+    if (dk % 4 == 0) TL_DELTA(bf16_t, true);
+    else TL_DELTA(bf16_t, false);
   }
-  int threads = (dv * lpc + kWave - 1) / kWave * kWave;
-  const size_t lds = ((size_t)kDeltaTile * (2 * dk + 2 * dv + 2)) * sizeof(float);
-  if (lds + 1024 > (size_t)tl_device_facts().lds_bytes)
-    return tl_fail(TL_ERR_UNSUPPORTED, "gated_delta: heads of %d by %d do not fit the LDS", dk, dv);
-  const dim3 grid(H, n_seqs);
-#define TL_DELTA(T, RB)                                                                                                  \
-  do {                                                                                                                   \
-    if (lds > 48 * 1024) {                                                                                               \
-      hipError_t e = hipFuncSetAttribute((const void*)gated_delta_kernel<T, RB>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
-      if (e != hipSuccess) return tl_fail(TL_ERR_HIP, "gated_delta: %s", hipGetErrorString(e));                          \
-    }                                                                                                                    \
-    gated_delta_kernel<T, RB><<<grid, threads, lds, stream>>>((const T*)qkv, qkv_stride, (const T*)proj, proj_stride, gate_off, \
-                                                              b_off, a_off, A_log, dt_bias, norm_w, eps, state, state_stride, \
-                                                              qo_indptr, slot_ids, (T*)out, H, G, dk, dv, lpc);          \
-  } while (0)
-#define TL_DELTA_RB(T)              \
-  do {                              \
-    if (rb == 16) TL_DELTA(T, 16);  \
-    else if (rb == 32) TL_DELTA(T, 32); \
-    else TL_DELTA(T, 64);           \
-  } while (0)
-  if (dtype == TL_F32) TL_DELTA_RB(float);
-  else if (dtype == TL_BF16) TL_DELTA_RB(bf16_t);
-  else return tl_fail(TL_ERR_ARG, "gated_delta: unknown dtype %d", dtype);
-#undef TL_DELTA_RB
 #undef TL_DELTA
-  return tl_check_launch("gated_delta");
+  int rc = tl_check_launch("gated_delta");
+  if (rc != TL_OK) return rc;
+  for (int t0 = 0; t0 < n_tokens; t0 += 65535) {
+    const int nt = n_tokens - t0 < 65535 ? n_tokens - t0 : 65535;
+    const dim3 ogrid(nt, (H + kHeadWaves - 1) / kHeadWaves);
+    const float* src = o_raw + (size_t)t0 * H * dv;
+    if (dtype == TL_F32)
+      delta_output_kernel<float><<<ogrid, kHeadWaves * kWave, 0, stream>>>(
+          src, (const float*)proj + (size_t)t0 * proj_stride, proj_stride, gate_off, norm_w, eps, (float*)out + (size_t)t0 * H * dv, H, dv);
+    else
+      delta_output_kernel<bf16_t><<<ogrid, kHeadWaves * kWave, 0, stream>>>(
+          src, (const bf16_t*)proj + (size_t)t0 * proj_stride, proj_stride, gate_off, norm_w, eps, (bf16_t*)out + (size_t)t0 * H * dv, H, dv);
+  }
+  return tl_check_launch("delta_output");
 }

@@ -39,8 +39,8 @@ _CORE_SIGNATURES = {
     "tl_gelu_mul": [_P, _P, _I, _I, _I, _P],
     "tl_rope_norm_kv_write": [_P, _I, _I, _I, _I, _I, _P, _I, _I, _F, _P, _P, _P, _I, _I, _P],
     "tl_causal_conv": [_P, _I, _P, _P, _P, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
-    "tl_selective_scan": [_P, _P, _I, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _P],
-    "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "tl_selective_scan": [_P, _P, _I, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P],
+    "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
     "tl_gemm_f32": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _P],

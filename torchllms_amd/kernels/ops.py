@@ -89,7 +89,9 @@ from .attention_ops import (  # noqa: F401
     prefill_tiles,
 )
 from .sequence_ops import (  # noqa: F401
+    SCAN_SEGMENTS_FROM,
     ScaledSum,
+    ScanSegments,
     causal_conv,
     embed_scaled,
     gated_delta,

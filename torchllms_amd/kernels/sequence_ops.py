@@ -203,6 +203,33 @@ def causal_conv(
     return out
 
 
+#: tokens of a segment when a long row's recurrence is cut into segments that run side by side, and the
+#: longest row of a step from which on that is done
+SCAN_SEGMENT = 64
+SCAN_SEGMENTS_FROM = 256
+
+
+class ScanSegments:
+    """The rows of a step cut into segments of at most ``SCAN_SEGMENT`` consecutive tokens: ``segs``
+    int32 [n, 2] (first token, one past the last) with every row's segments in order, ``row_seg`` int32
+    [rows + 1] (the first segment of every row), both on the device, made from the host's row offsets."""
+
+    def __init__(self, qo_indptr_host, device, length: int = SCAN_SEGMENT):
+        import numpy as np
+
+        bounds = [int(v) for v in qo_indptr_host]
+        segs, row_seg = [], [0]
+        for lo, hi in zip(bounds[:-1], bounds[1:]):
+            for t in range(lo, hi, length):
+                segs.append((t, min(t + length, hi)))
+            row_seg.append(len(segs))
+        self.n = len(segs)
+        packed = np.asarray([v for seg in segs for v in seg] + row_seg, dtype=np.int32)
+        dev = torch.from_numpy(packed).to(device)
+        self.segs = dev[: 2 * self.n]
+        self.row_seg = dev[2 * self.n :]
+
+
 def selective_scan(
     x: torch.Tensor,
     dt_pre: torch.Tensor,
@@ -217,13 +244,17 @@ def selective_scan(
     state_offset: int,
     qo_indptr: torch.Tensor,
     slot_ids: torch.Tensor,
+    segments: Optional[ScanSegments] = None,
 ) -> torch.Tensor:
     """The recurrence of a diagonal state-space layer over each request's tokens, in 32-bit:
     ``dt = softplus(dt_pre + dt_bias)``; ``S[c, n] = exp(dt[c] A[c, n]) S[c, n] + dt[c] x[c] B[n]``;
     ``y[c] = sum_n S[c, n] C[n] + D[c] x[c]``; result ``y * silu(z)``.  ``x`` [n, inner]; ``dt_pre``
     [n, inner] (32-bit or x's dtype); B and C are the ``N`` columns of ``proj`` from ``b_offset`` and
     ``c_offset``; ``z`` [n, inner] may be a view of columns; ``A`` float32 [inner, N] (negative);
-    ``S`` lives at ``state_offset`` of the request's state row, inner * N floats."""
+    ``S`` lives at ``state_offset`` of the request's state row, inner * N floats.  With ``segments`` the
+    rows' segments run side by side: each is walked from a zero state, a carry joins the segments of a
+    row in order (a state's decay over a segment is exp(A * the sum of the segment's step sizes)), and
+    each is walked again from the state that enters it.  The result then depends on the cut by rounding."""
     _gpu(x, dt_pre, proj, z, dt_bias, A, D)
     n, inner = x.shape
     N = A.shape[1]
@@ -239,11 +270,19 @@ def selective_scan(
     n_seqs = _step_rows(None, qo_indptr, slot_ids, n, state)
     region, stride = state_region(state, state_offset, inner * N)
     out = torch.empty_like(x)
+    ws = seg_dt = None
+    if segments is not None:
+        if segments.row_seg.numel() != n_seqs + 1:
+            raise KernelError("selective_scan: the segments are not those of this step's rows")
+        ws = torch.empty((segments.n, inner * N), dtype=torch.float32, device=x.device)
+        seg_dt = torch.empty((segments.n, inner), dtype=torch.float32, device=x.device)
     check(
         core().tl_selective_scan(
             x.data_ptr(), dt_pre.data_ptr(), dtype_code(dt_pre.dtype), proj.data_ptr(), proj.stride(0), b_offset, c_offset,
             z.data_ptr(), z.stride(0), dt_bias.data_ptr(), A.data_ptr(), D.data_ptr(), region, stride, qo_indptr.data_ptr(),
-            slot_ids.data_ptr(), out.data_ptr(), n_seqs, inner, N, dtype_code(x.dtype), _stream(),
+            slot_ids.data_ptr(), out.data_ptr(), n_seqs, inner, N, dtype_code(x.dtype),
+            _ptr(segments.segs) if segments is not None else None, _ptr(segments.row_seg) if segments is not None else None,
+            segments.n if segments is not None else 0, _ptr(ws), _ptr(seg_dt), _stream(),
         )
     )
     return out
@@ -290,11 +329,12 @@ def gated_delta(
     n_seqs = _step_rows(None, qo_indptr, slot_ids, n, state)
     region, stride = state_region(state, state_offset, H * dv * dk)
     out = torch.empty((n, H * dv), dtype=qkv.dtype, device=qkv.device)
+    o_raw = torch.empty((n, H * dv), dtype=torch.float32, device=qkv.device)
     check(
         core().tl_gated_delta(
             qkv.data_ptr(), qkv.stride(0), proj.data_ptr(), proj.stride(0), gate_offset, b_offset, a_offset, A_log.data_ptr(),
             dt_bias.data_ptr(), norm_weight.data_ptr(), float(eps), region, stride, qo_indptr.data_ptr(), slot_ids.data_ptr(),
-            out.data_ptr(), n_seqs, H, G, dk, dv, dtype_code(qkv.dtype), _stream(),
+            out.data_ptr(), n, n_seqs, H, G, dk, dv, o_raw.data_ptr(), dtype_code(qkv.dtype), _stream(),
         )
     )
     return out

@@ -73,12 +73,20 @@ class SelectiveScan(Mixer):
     def forward(self, x, ctx, cache):
         c, n, r = self.inner, self.n_state, self.dt_rank
         state = cache.tensor
-        xz = ops.linear(ops.resolved(x), self.w_in)
+        x = ops.resolved(x)
+        xz = ops.linear(x, self.w_in)
         xc = ops.causal_conv(xz[:, :c], self.conv_w, self.conv_b, state, 0, ctx.token_seq, ctx.qo_indptr, ctx.slot_ids)
         proj = ops.linear(xc, self.w_x)
         dt_pre = ops.linear(proj[:, :r], self.w_dt, out_dtype=torch.float32)
+        # a long prompt's recurrence is cut into segments that run side by side; in 32-bit every row is
+        # walked in one piece, so that no bit depends on how the prompt was cut into steps
+        segments = None
+        if x.dtype != torch.float32 and ctx.host.max_q_len >= ops.SCAN_SEGMENTS_FROM:
+            segments = ctx.scratch.get("scan_segments")
+            if segments is None:
+                segments = ctx.scratch["scan_segments"] = ops.ScanSegments(ctx.host.qo_indptr, x.device)
         y = ops.selective_scan(xc, dt_pre, proj, r, r + n, xz[:, c:], self.dt_b, self.A, self.D, state, (self.taps - 1) * c,
-                               ctx.qo_indptr, ctx.slot_ids)
+                               ctx.qo_indptr, ctx.slot_ids, segments=segments)
         return ops.linear_to_sum(y, self.w_o)
 
 
@@ -120,8 +128,8 @@ class GatedDelta(Mixer):
         }
 
     def check_sizes(self, dtype: torch.dtype) -> None:
-        if self.dk > 1024 or self.dv > 1024 or self.dk * self.dv > 256 * 256:
-            raise ValueError(f"gated_delta: heads of {self.dk} by {self.dv}; the kernel takes up to 256 by 256")
+        if self.dk > 256:
+            raise ValueError(f"gated_delta: keys of {self.dk} channels; the kernel takes up to 256 (values: any number)")
         if self.taps > 64:
             raise ValueError(f"gated_delta: a convolution over {self.taps} taps; the kernel takes up to 64")
 
