@@ -119,6 +119,10 @@ ALONE = {
     "attention": models.layer("attention", models.attention(4, 2, 32, 48, 20, 16, 0.25, 6.0)),
     "attention_whole_head_rotated": models.layer("attention", models.attention(3, 3, 16, 16, 16, 9, 0.5, 30.0,
                                                  scaling={"factor": 4.0, "low": 1.0, "high": 4.0, "original": 16})),
+    # keys and values of one head size that the matrix-core attention kernels take (bfloat16 runs those), with a
+    # cap low enough to bend most scores
+    "attention_matrix_cores_64": models.layer("attention", models.attention(8, 2, 64, 64, 32, 48, 0.6, 4.0)),
+    "attention_matrix_cores_128": models.layer("attention", models.attention(4, 1, 128, 128, 64, 100, 0.4, 5.0, base=300.0)),
     "delta": models.layer("delta", {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 40, "conv": 4}),
     "delta_wide": models.layer("delta", {"heads": 1, "kv_heads": 1, "dim": 256, "vdim": 64, "conv": 2}),
     "delta_odd": models.layer("delta", {"heads": 3, "kv_heads": 1, "dim": 18, "vdim": 70, "conv": 3}),
@@ -137,14 +141,14 @@ def test_a_mechanism_alone(tmp_path, what, dtype):
 
     folder = models.make_folder(tmp_path / what, models.single_layer(ALONE[what]), seed=5)
     cfg, weights = models.read_folder(folder)
-    tokens = random_tokens(75, cfg["vocab"], 9)
+    tokens = random_tokens(275, cfg["vocab"], 9)
     truth, scale = truth_of(cfg, weights, {"r": tokens})
-    engine = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=24, max_seqs=2)
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=80, max_seqs=2)
     engine.admit("whole")
     whole = engine.step([StepEntry("whole", tokens, list(range(len(tokens))))]).cpu()
     engine.admit("cut")
     rows, at = [], 0
-    for n in (5, 2, 30, 1, 1, 1, 17, 2, 1, 1, 13, 1):
+    for n in (5, 2, 30, 1, 1, 1, 17, 2, 1, 1, 13, 1, 150, 1, 1, 47, 1):
         rows.append(engine.step([StepEntry("cut", tokens[at : at + n], list(range(n)))]).cpu())
         at += n
     assert at == len(tokens)

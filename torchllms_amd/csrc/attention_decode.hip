@@ -76,12 +76,23 @@ struct DecodeArgs {
   int page_size;
   int page_shift;  // log2(page_size) when that is a power of two, else -1
   int window;
+  int chunk;          // > 0: a query sees only the keys of its own chunk of that many positions
   float scale_log2e;  // softmax scale * log2(e): probabilities are exp2 of scaled differences
+  float cap_log2e;    // > 0: scores are capped, cap * tanh(score / cap); this is cap * log2(e) ...
+  float two_scale_over_cap_log2e;  // ... and this 2 * scale / cap * log2(e): tanh(x) = 1 - 2 / (exp2(2 x log2(e)) + 1)
+  const float* sinks;  // per query head, or null: exp(sink) joins the softmax's denominator
   int split_size;     // keys per split, a multiple of 64
   int n_splits;
   float* ws_o;   // [token][q head][split][DH]
   float* ws_ml;  // [token][q head][split][2] = running maximum (log2 domain), sum
 };
+
+// The first position a query at p sees: behind its window, inside its chunk.
+__device__ __forceinline__ int first_key(int p, int window, int chunk) {
+  int lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
+  if (chunk > 0) lo = max(lo, p - p % chunk);
+  return lo;
+}
 
 struct Pack16 {
   u32x4_t u;
@@ -137,7 +148,7 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
 
   const int b = a.token_seq[t];
   const int p = a.positions[t];
-  const int lo = (a.window > 0 && p - a.window + 1 > 0) ? p - a.window + 1 : 0;
+  const int lo = first_key(p, a.window, a.chunk);
   const int lo_al = lo & ~(kTile - 1);
   const int split_begin = lo_al + split * a.split_size;
   if (split_begin > p) return;  // whole block: nothing in this split
@@ -238,7 +249,10 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
     for (int i = 0; i < 4; ++i) {
       const int key = base + 4 * g4 + i;
       const bool valid = (key >= lo) & (key <= p);  // bit operation: no branch behind the MFMAs
-      s[i] = valid ? c[i] * a.scale_log2e : -INFINITY;
+      float sc = c[i] * a.scale_log2e;
+      if (a.cap_log2e > 0.f)  // (the same in every lane)
+        sc = a.cap_log2e * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(c[i] * a.two_scale_over_cap_log2e) + 1.0f));
+      s[i] = valid ? sc : -INFINITY;
       tmax = fmaxf(tmax, s[i]);
     }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
@@ -301,6 +315,7 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
     }
     const int qh = kvh * R + h;
     if (a.n_splits == 1) {
+      if (a.sinks) L += __builtin_amdgcn_exp2f(a.sinks[qh] * 1.4426950408889634f - M);
       a.out[(size_t)t * a.out_stride + (size_t)qh * DH + d] = from_f32<bf16_t>(O / L);
     } else {
       const size_t slot = ((size_t)t * a.n_kv_heads * R + qh) * a.n_splits + split;
@@ -343,7 +358,7 @@ __global__ void __launch_bounds__(kWave) attn_decode_merge_kernel(DecodeArgs a, 
     }
   };
   fetch(0);
-  const int lo = (a.window > 0 && p - a.window + 1 > 0) ? p - a.window + 1 : 0;
+  const int lo = first_key(p, a.window, a.chunk);
   const int lo_al = lo & ~(kTile - 1);
   const int n_valid = min((p - lo_al) / a.split_size + 1, a.n_splits);
   float M = lane < n_valid ? m_mine : -INFINITY;
@@ -353,6 +368,7 @@ __global__ void __launch_bounds__(kWave) attn_decode_merge_kernel(DecodeArgs a, 
   for (int s = lane + kWave; s < n_valid; s += kWave)
     L += a.ws_ml[(slot0 + s) * 2 + 1] * __builtin_amdgcn_exp2f(a.ws_ml[(slot0 + s) * 2] - M);
   L = wave_sum(L);
+  if (a.sinks) L += __builtin_amdgcn_exp2f(a.sinks[qh] * 1.4426950408889634f - M);
   float o[NC];
 #pragma unroll
   for (int c = 0; c < NC; ++c) o[c] = 0.f;
@@ -380,16 +396,18 @@ __global__ void __launch_bounds__(kWave) attn_decode_merge_kernel(DecodeArgs a, 
 TL_EXPORT int tl_attn_decode_head_dim() { return DH; }
 
 // q: element (t, h, d) at q + t*q_stride + h*DH + d; out likewise.  Pages [page][Hkv][page_size][DH].
-// Every token is one query at positions[t] of request row token_seq[t].  split_size: keys per
+// softcap > 0 caps the scores, chunk > 0 confines a query to its chunk, sinks (one float per query head, or
+// null) join the denominators.  Every token is one query at positions[t] of request row token_seq[t].  split_size: keys per
 // split (a multiple of 64); n_splits >= ceil(longest visible range / split_size), counted from the
 // 16-aligned first visible key.  ws_o / ws_ml: workspaces (unused when n_splits == 1).
 TL_EXPORT int tl_attn_decode(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                              const void* v_pages, const int32_t* token_seq, const int32_t* positions,
                              const int32_t* block_table, int bt_stride, int n_tokens, int n_q_heads,
                              int n_kv_heads, int head_dim, int page_size, int window, float scale,
-                             int split_size, int n_splits, float* ws_o, float* ws_ml, hipStream_t stream) {
+                             int split_size, int n_splits, float* ws_o, float* ws_ml, float softcap, int chunk,
+                             const float* sinks, hipStream_t stream) {
   if (head_dim != DH) return variant_fail(TL_ERR_ARG, "attn_decode: built for head_dim %d, called with %d", DH, head_dim);
-  if (n_tokens < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || page_size <= 0 || bt_stride <= 0 || window < 0)
+  if (n_tokens < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || page_size <= 0 || bt_stride <= 0 || window < 0 || chunk < 0 || softcap < 0)
     return variant_fail(TL_ERR_ARG, "attn_decode: bad sizes");
   if (n_q_heads % n_kv_heads) return variant_fail(TL_ERR_ARG, "attn_decode: %d query heads are not a multiple of %d kv heads", n_q_heads, n_kv_heads);
   const int R = n_q_heads / n_kv_heads;
@@ -409,6 +427,9 @@ TL_EXPORT int tl_attn_decode(const void* q, int q_stride, void* out, int out_str
   for (int sh = 0; sh < 31; ++sh)
     if ((1 << sh) == page_size) a.page_shift = sh;
   a.scale_log2e = scale * 1.4426950408889634f;
+  a.chunk = chunk; a.sinks = sinks;
+  a.cap_log2e = softcap > 0 ? softcap * 1.4426950408889634f : 0.f;
+  a.two_scale_over_cap_log2e = softcap > 0 ? 2.0f * scale / softcap * 1.4426950408889634f : 0.f;
   a.split_size = split_size; a.n_splits = n_splits; a.ws_o = ws_o; a.ws_ml = ws_ml;
   dim3 grid(n_splits, n_kv_heads, n_tokens);
   const int threads = kWaves * kWave;

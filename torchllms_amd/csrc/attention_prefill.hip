@@ -98,7 +98,11 @@ struct PrefillArgs {
   int page_size;
   int page_shift;  // log2(page_size)
   int window;
+  int chunk;  // > 0: a query sees only the keys of its own chunk of that many positions
   float scale_log2e;
+  float cap_over_scale;             // capped scores: s <- cap * tanh(s * scale / cap), taken on the raw product as
+  float two_scale_over_cap_log2e;   // c <- (cap / scale) * (1 - 2 / (exp2(c * 2 scale / cap * log2(e)) + 1))
+  const float* sinks;               // per query head, or null: exp(sink) joins the softmax's denominator
 };
 
 typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
@@ -154,8 +158,10 @@ __device__ __forceinline__ u32x2_t lds_transposed(const bf16_t* src) {
 // of kWaves waves that take the same columns and every second tile of keys each, and add up what
 // they have at the end through LDS: a block's chain of tiles is half as long, which is what a launch
 // needs whose blocks all fit the GPU at once and whose time is therefore that of its longest block.
-template <int RP, bool WINDOWED, int GROUPS>
+// MODE 0: no lower bound and no cap; 1: a lower bound (a window, chunks, or both); 2: a lower bound and capped scores.
+template <int RP, int MODE, int GROUPS>
 __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) attn_prefill_kernel(PrefillArgs a) {
+  constexpr bool WINDOWED = MODE >= 1, CAPPED = MODE == 2;
   constexpr int QB = kCols / RP;  // queries per block
 
   const int tile = blockIdx.y;  // the host lists the tiles in the order that balances the launch
@@ -177,7 +183,11 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
   const int32_t* bt = a.block_table + (size_t)row * a.bt_stride;
   const size_t head_elems = (size_t)a.page_size * DH;
 
-  auto window_lo = [&](int pos) { return (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0; };
+  auto window_lo = [&](int pos) {
+    int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+    if (a.chunk > 0) lo = max(lo, pos - pos % a.chunk);
+    return lo;
+  };
   const int q_last = min(q0 + QB, q_len) - 1;       // last query of the tile
   const int key_lo = window_lo(pos0 + q0);          // first key any column sees
   const int key_hi = pos0 + q_last;                 // last key any column sees
@@ -432,6 +442,15 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
     // a tile that lies wholly before the block's first query (and behind every window's edge) is seen
     // whole by every column: no masks (the same decision for all waves of the block)
     const int base = base_of(step);
+    if constexpr (CAPPED) {
+#pragma unroll
+      for (int i = 0; i < NC; ++i)
+#pragma unroll
+        for (int sub = 0; sub < NS; ++sub)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            c[i][sub][r] = a.cap_over_scale * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(c[i][sub][r] * a.two_scale_over_cap_log2e) + 1.0f));
+    }
     if (base + KT - 1 > pos0 + q0 || (WINDOWED && base < window_lo(pos0 + q_last))) mask(base);
     softmax(pb, alpha, moved);
     output(v_tile(step - 1), pb_prev);
@@ -488,6 +507,7 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
       const float mine = m_run[i] == -INFINITY ? 0.f : exp2_fast(m_run[i] - m_new);
       const float other = m_other == -INFINITY ? 0.f : exp2_fast(m_other - m_new);
       l_part[i] = l_part[i] * mine + x[kStride] * other;
+      m_run[i] = m_new;
 #pragma unroll
       for (int t = 0; t < DT; ++t)
 #pragma unroll
@@ -497,8 +517,9 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
 
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
-    const float l = l_part[i];
+    float l = l_part[i];
     if (!col_ok[i]) continue;
+    if (a.sinks) l += exp2_fast(a.sinks[col_head[i]] * 1.4426950408889634f - m_run[i]);
     const float inv = 1.0f / l;
     bf16_t* orow = a.out + (size_t)col_tok[i] * a.out_stride + (size_t)col_head[i] * DH;
     // acc[i][t][r] is channel 16 t + 4 g4 + r: four consecutive channels per output block
@@ -524,9 +545,10 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
                               const void* v_pages, const int32_t* qo_indptr, const int32_t* kv_lens,
                               const int32_t* block_table, int bt_stride, const int32_t* tile_row,
                               const int32_t* tile_q0, int n_tiles, int n_q_heads, int n_kv_heads, int head_dim,
-                              int page_size, int window, float scale, int key_groups, hipStream_t stream) {
+                              int page_size, int window, float scale, int key_groups, float softcap, int chunk,
+                              const float* sinks, hipStream_t stream) {
   if (head_dim != DH) return variant_fail(TL_ERR_ARG, "attn_prefill: built for head_dim %d, called with %d", DH, head_dim);
-  if (n_tiles < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || page_size <= 0 || bt_stride <= 0 || window < 0)
+  if (n_tiles < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || page_size <= 0 || bt_stride <= 0 || window < 0 || chunk < 0 || softcap < 0)
     return variant_fail(TL_ERR_ARG, "attn_prefill: bad sizes");
   if (n_q_heads % n_kv_heads) return variant_fail(TL_ERR_ARG, "attn_prefill: %d query heads are not a multiple of %d kv heads", n_q_heads, n_kv_heads);
   const int R = n_q_heads / n_kv_heads;
@@ -553,17 +575,22 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
     return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: pages of %d tokens are shorter than the %d rows a wave fetches at once at head size %d",
                         page_size, kRowsPerLoad, DH);
   a.scale_log2e = scale * 1.4426950408889634f;
+  a.chunk = chunk; a.sinks = sinks;
+  a.cap_over_scale = softcap > 0 ? softcap / scale : 0.f;
+  a.two_scale_over_cap_log2e = softcap > 0 ? 2.0f * scale / softcap * 1.4426950408889634f : 0.f;
   dim3 grid(n_kv_heads, n_tiles);  // consecutive blocks share a query tile: their loads of q overlap
-  const bool windowed = window > 0;
+  const int mode = softcap > 0 ? 2 : (window > 0 || chunk > 0) ? 1 : 0;
   const int threads = kWaves * kWave;
 #define TL_PREFILL_LAUNCH(rp)                                                                      \
   do {                                                                                             \
     if (key_groups == 2) {                                                                         \
-      if (windowed) attn_prefill_kernel<rp, true, 2><<<grid, 2 * threads, 0, stream>>>(a);         \
-      else attn_prefill_kernel<rp, false, 2><<<grid, 2 * threads, 0, stream>>>(a);                 \
+      if (mode == 2) attn_prefill_kernel<rp, 2, 2><<<grid, 2 * threads, 0, stream>>>(a);           \
+      else if (mode == 1) attn_prefill_kernel<rp, 1, 2><<<grid, 2 * threads, 0, stream>>>(a);      \
+      else attn_prefill_kernel<rp, 0, 2><<<grid, 2 * threads, 0, stream>>>(a);                     \
     } else {                                                                                       \
-      if (windowed) attn_prefill_kernel<rp, true, 1><<<grid, threads, 0, stream>>>(a);             \
-      else attn_prefill_kernel<rp, false, 1><<<grid, threads, 0, stream>>>(a);                     \
+      if (mode == 2) attn_prefill_kernel<rp, 2, 1><<<grid, threads, 0, stream>>>(a);               \
+      else if (mode == 1) attn_prefill_kernel<rp, 1, 1><<<grid, threads, 0, stream>>>(a);          \
+      else attn_prefill_kernel<rp, 0, 1><<<grid, threads, 0, stream>>>(a);                         \
     }                                                                                              \
   } while (0)
   if (R == 1) TL_PREFILL_LAUNCH(1);

@@ -203,26 +203,42 @@ rope_norm_kv_write_kernel(T* qkv, int row, int n_q, int n_kv, int dk, int dv, co
 // hist[k][c] at state + slot * state_stride + k * C + c, oldest first, zero for a new request.
 //   out[t, c] = act(bias[c] + sum_j taps[c][j] * in(t - (K - 1 - j))),  j ascending, 32-bit
 // act 0: none, 1: silu.  The history is brought up to date by a second kernel, after every token has read it.
-template <typename T>
+template <typename T, int V>
 __global__ void __launch_bounds__(256)
 causal_conv_kernel(const T* __restrict__ x, int x_stride, const float* __restrict__ taps, const float* __restrict__ bias,
                    const float* __restrict__ state, long long state_stride, const int32_t* __restrict__ token_seq,
                    const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ slot_ids, T* __restrict__ out,
                    int out_stride, int C, int K, int act, int t0) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  // a thread takes V neighbouring channels of one token (V elements = 16 bytes where the rows allow it)
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * V;
   if (c >= C) return;
   const int t = t0 + blockIdx.y;
   const int row = token_seq[t];
   const int start = qo_indptr[row];
   const int i = t - start;
   const float* hist = state + (long long)slot_ids[row] * state_stride;
-  float acc = bias ? bias[c] : 0.f;
+  struct alignas(sizeof(T) * V) Vec { T e[V]; };
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = bias ? bias[c + e] : 0.f;
   for (int j = 0; j < K; ++j) {
     const int src = i - (K - 1 - j);
-    const float v = src >= 0 ? to_f32(x[(size_t)(start + src) * x_stride + c]) : hist[(size_t)(K - 1 + src) * C + c];
-    acc = fmaf(taps[(size_t)c * K + j], v, acc);
+    float v[V];
+    if (src >= 0) {
+      const Vec in = *reinterpret_cast<const Vec*>(x + (size_t)(start + src) * x_stride + c);
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = to_f32(in.e[e]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = hist[(size_t)(K - 1 + src) * C + c + e];
+    }
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = fmaf(taps[(size_t)(c + e) * K + j], v[e], acc[e]);
   }
-  out[(size_t)t * out_stride + c] = from_f32<T>(act == 1 ? silu_f(acc) : acc);
+  Vec o;
+#pragma unroll
+  for (int e = 0; e < V; ++e) o.e[e] = from_f32<T>(act == 1 ? silu_f(acc[e]) : acc[e]);
+  *reinterpret_cast<Vec*>(out + (size_t)t * out_stride + c) = o;
 }
 
 // New history of every request of the step: the last K - 1 entries of (old history, the step's inputs).
@@ -291,6 +307,16 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
   float dt_sum = 0.f;
   for (int t0 = start; t0 < end; t0 += kScanTile) {
     const int nt = min(kScanTile, end - t0);
+    // the tile's own inputs are asked for at once, before anything waits for one of them
+    T x_t[kScanTile], z_t[kScanTile];
+    DT dt_t[kScanTile];
+#pragma unroll
+    for (int tt = 0; tt < kScanTile; ++tt) {
+      const size_t t = (size_t)(t0 + (tt < nt ? tt : 0));
+      x_t[tt] = x[t * inner + c];
+      dt_t[tt] = dt_pre[t * inner + c];
+      if (MODE != 1) z_t[tt] = z[t * z_stride + c];
+    }
     __syncthreads();  // everybody has finished with the tile before
     for (int idx = threadIdx.x; idx < nt * 2 * N; idx += kScanThreads) {
       const int tt = idx / (2 * N), e = idx % (2 * N);
@@ -298,11 +324,13 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
       bc_lds[idx] = to_f32(e < N ? src[b_off + e] : src[c_off + e - N]);
     }
     __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
+#pragma unroll
+    for (int tt = 0; tt < kScanTile; ++tt) {
+      if (tt >= nt) break;
       const size_t t = (size_t)(t0 + tt);
-      const float xv = to_f32(x[t * inner + c]);
-      const float dt = softplus_f(to_f32(dt_pre[t * inner + c]) + bias);
-      const float zv = MODE == 1 ? 0.f : to_f32(z[t * z_stride + c]);
+      const float xv = to_f32(x_t[tt]);
+      const float dt = softplus_f(to_f32(dt_t[tt]) + bias);
+      const float zv = MODE == 1 ? 0.f : to_f32(z_t[tt]);
       const float dx = dt * xv;
       dt_sum += dt;
       const float* Bt = bc_lds + tt * 2 * N + n0;
@@ -405,9 +433,11 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
                    int col_groups) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // per token of the tile: k [dk], q [dk] (raw, then unit), v [kDeltaCols], o [kDeltaCols]; then beta, decay, 1/|k|, scale/|q|
+  const int dkp = dk + dk / 16 * 4;  // a token's keys in LDS: four floats of padding after every sixteen, so that
+                                     // the lanes of a column, sixteen rows apart, read different banks
   float* k_l = lds;
-  float* q_l = k_l + kDeltaTile * dk;
-  float* v_l = q_l + kDeltaTile * dk;
+  float* q_l = k_l + kDeltaTile * dkp;
+  float* v_l = q_l + kDeltaTile * dkp;
   float* o_l = v_l + kDeltaTile * kDeltaCols;
   float* sc_l = o_l + kDeltaTile * kDeltaCols;  // [kDeltaTile][4]
   const int row = blockIdx.y;
@@ -422,8 +452,16 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
   const int i0 = part * kDeltaRows;
   float* st = state + (long long)slot_ids[row] * state_stride + ((size_t)h * dv + j) * dk;
   float S[kDeltaRows];
+  if (VEC) {
 #pragma unroll
-  for (int r = 0; r < kDeltaRows; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
+    for (int r = 0; r < kDeltaRows; r += 4) {
+      const float4 s4 = i0 + r < dk ? *reinterpret_cast<const float4*>(st + i0 + r) : float4{0.f, 0.f, 0.f, 0.f};
+      S[r] = s4.x; S[r + 1] = s4.y; S[r + 2] = s4.z; S[r + 3] = s4.w;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < kDeltaRows; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
+  }
   const float neg_rate = -expf(A_log[h]), bias = dt_bias[h];
   const float q_scale = 1.0f / sqrtf((float)dk);
   const int q_col = g * dk, k_col = G * dk + g * dk, v_col = 2 * G * dk + h * dv + cg * kDeltaCols;
@@ -432,9 +470,14 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
   // what a thread fetches of a tile: element e of the tile's keys and queries (e = tt * 2 dk + d, d < dk a
   // key's channel, else a query's) for e = tid, tid + threads, ...; likewise of the values
   constexpr int kPreKQ = 16, kPreV = 8;
-  T pre_kq[kPreKQ], pre_v[kPreV];
+  T pre_kq[kPreKQ], pre_v[kPreV], pre_b = from_f32<T>(0.f), pre_a = from_f32<T>(0.f);
   auto fetch = [&](int t0) {
     const int nt = min(kDeltaTile, end - t0);
+    if (threadIdx.x < nt) {
+      const T* pr = proj + (size_t)(t0 + threadIdx.x) * proj_stride;
+      pre_b = pr[b_off + h];
+      pre_a = pr[a_off + h];
+    }
 #pragma unroll
     for (int u = 0; u < kPreKQ; ++u) {
       const int e = threadIdx.x + u * n_threads;
@@ -456,7 +499,8 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
     for (int u = 0; u < kPreKQ; ++u) {
       const int e = threadIdx.x + u * n_threads;
       const int tt = e / (2 * dk), d = e % (2 * dk);
-      if (tt < nt) (d < dk ? k_l[tt * dk + d] : q_l[tt * dk + d - dk]) = to_f32(pre_kq[u]);
+      const int dd = d < dk ? d : d - dk;
+      if (tt < nt) (d < dk ? k_l : q_l)[tt * dkp + dd + dd / 16 * 4] = to_f32(pre_kq[u]);
     }
 #pragma unroll
     for (int u = 0; u < kPreV; ++u) {
@@ -465,31 +509,38 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
       if (tt < nt && d < v_cols) v_l[tt * kDeltaCols + d] = to_f32(pre_v[u]);
     }
     if (threadIdx.x < nt) {
-      const T* pr = proj + (size_t)(t0 + threadIdx.x) * proj_stride;
-      sc_l[4 * threadIdx.x] = sigmoid_f(to_f32(pr[b_off + h]));
-      sc_l[4 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pr[a_off + h]) + bias));
+      sc_l[4 * threadIdx.x] = sigmoid_f(to_f32(pre_b));
+      sc_l[4 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pre_a) + bias));
     }
     if (t0 + kDeltaTile < end) fetch(t0 + kDeltaTile);  // on its way while this tile is worked on
     __syncthreads();
-    // the norms: 2 nt vectors, each summed by one thread in ascending order of its channels
-    if (threadIdx.x < 2 * nt) {
-      const int tt = threadIdx.x / 2, which = threadIdx.x % 2;
-      const float* src = (which ? q_l : k_l) + tt * dk;
+    // the norms: 2 nt vectors, each summed by eight neighbouring lanes (a lane its channels in ascending
+    // order, the lanes by moves in a fixed order); every thread of the first waves takes part in the moves
+    for (int v0 = 0; v0 < 2 * kDeltaTile; v0 += n_threads / 8) {
+      const int vec = v0 + threadIdx.x / 8, sub = threadIdx.x % 8;
+      const int tt = vec / 2, which = vec % 2;
       float ss = 0.f;
-      for (int d = 0; d < dk; ++d) ss = fmaf(src[d], src[d], ss);
-      sc_l[4 * tt + 2 + which] = (which ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
+      if (tt < nt) {
+        const float* src = (which ? q_l : k_l) + tt * dkp;
+        for (int d = sub; d < dk; d += 8) {
+          const float e = src[d + d / 16 * 4];
+          ss = fmaf(e, e, ss);
+        }
+      }
+      ss = row_group_sum(ss, 8);
+      if (tt < nt && sub == 0) sc_l[4 * tt + 2 + which] = (which ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
     }
     __syncthreads();
     for (int e = threadIdx.x; e < nt * 2 * dk; e += n_threads) {
       const int tt = e / (2 * dk), d = e % (2 * dk);
-      if (d < dk) k_l[tt * dk + d] *= sc_l[4 * tt + 2];
-      else q_l[tt * dk + d - dk] *= sc_l[4 * tt + 3];
+      const int dd = d < dk ? d : d - dk;
+      (d < dk ? k_l : q_l)[tt * dkp + dd + dd / 16 * 4] *= sc_l[4 * tt + (d < dk ? 2 : 3)];
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
       const float beta = sc_l[4 * tt], decay = sc_l[4 * tt + 1];
-      const float* kt = k_l + tt * dk + i0;
-      const float* qt = q_l + tt * dk + i0;
+      const float* kt = k_l + tt * dkp + i0 + i0 / 16 * 4;  // (i0 is a multiple of 16: a lane's rows have no padding between them)
+      const float* qt = q_l + tt * dkp + i0 + i0 / 16 * 4;
       float kk[kDeltaRows], qq[kDeltaRows];
       if (VEC) {  // dk is a multiple of 4: four channels a read
 #pragma unroll
@@ -531,9 +582,15 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
     }
   }
   if (live) {
+    if (VEC) {
 #pragma unroll
-    for (int r = 0; r < kDeltaRows; ++r)
-      if (i0 + r < dk) st[i0 + r] = S[r];
+      for (int r = 0; r < kDeltaRows; r += 4)
+        if (i0 + r < dk) *reinterpret_cast<float4*>(st + i0 + r) = float4{S[r], S[r + 1], S[r + 2], S[r + 3]};
+    } else {
+#pragma unroll
+      for (int r = 0; r < kDeltaRows; ++r)
+        if (i0 + r < dk) st[i0 + r] = S[r];
+    }
   }
 }
 
@@ -634,17 +691,23 @@ TL_EXPORT int tl_causal_conv(const void* x, int x_stride, const float* taps, con
   if (n_tokens == 0) return TL_OK;
   if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "causal_conv: unknown dtype %d", dtype);
   const int cblocks = (C + 255) / 256;
+  const int elt = dtype == TL_F32 ? 4 : 2, vec = 16 / elt;
+  const bool wide = C % vec == 0 && x_stride % vec == 0 && out_stride % vec == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0;
+  const int vblocks = (C / (wide ? vec : 1) + 255) / 256;
   for (int t0 = 0; t0 < n_tokens; t0 += 65535) {
     const int nt = n_tokens - t0 < 65535 ? n_tokens - t0 : 65535;
-    const dim3 grid(cblocks, nt);
-    if (dtype == TL_F32)
-      causal_conv_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_stride, taps, bias, state, state_stride,
-                                                          token_seq, qo_indptr, slot_ids, (float*)out, out_stride, C, K,
-                                                          act, t0);
-    else
-      causal_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_stride, taps, bias, state, state_stride,
-                                                           token_seq, qo_indptr, slot_ids, (bf16_t*)out, out_stride, C, K,
-                                                           act, t0);
+    const dim3 grid(vblocks, nt);
+#define TL_CONV(T, V)                                                                                                  \
+  causal_conv_kernel<T, V><<<grid, 256, 0, stream>>>((const T*)x, x_stride, taps, bias, state, state_stride, token_seq, \
+                                                     qo_indptr, slot_ids, (T*)out, out_stride, C, K, act, t0)
+    if (dtype == TL_F32) {
+      if (wide) TL_CONV(float, 4);
+      else TL_CONV(float, 1);
+    } else {
+      if (wide) TL_CONV(bf16_t, 8);
+      else TL_CONV(bf16_t, 1);
+    }
+#undef TL_CONV
   }
   int rc = tl_check_launch("causal_conv");
   if (rc != TL_OK || K == 1 || n_seqs == 0) return rc;
@@ -739,17 +802,19 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
   while (kDeltaRows * lpc < dk) lpc *= 2;  // at most 16: a column's lanes lie in one row of 16 lanes
   const int threads = (kDeltaCols * lpc + kWave - 1) / kWave * kWave;
   const int col_groups = (dv + kDeltaCols - 1) / kDeltaCols;
-  const size_t lds = ((size_t)kDeltaTile * (2 * dk + 2 * kDeltaCols + 4)) * sizeof(float);
+  const size_t lds = ((size_t)kDeltaTile * (2 * (dk + dk / 16 * 4) + 2 * kDeltaCols + 4)) * sizeof(float);
   const dim3 grid(H * col_groups, n_seqs);
 #define TL_DELTA(T, VEC)                                                                                               \
   gated_delta_kernel<T, VEC><<<grid, threads, lds, stream>>>((const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, \
                                                              a_off, A_log, dt_bias, state, state_stride, qo_indptr, slot_ids, \
                                                              o_raw, H, G, dk, dv, lpc, col_groups)
+  // four rows a load where every lane's rows start at a multiple of 16 bytes, in LDS and in the state
+  const bool vec = dk % 4 == 0 && ((uintptr_t)state % 16) == 0 && state_stride % 4 == 0;
   if (dtype == TL_F32) {
-    if (dk % 4 == 0) TL_DELTA(float, true);
+    if (vec) TL_DELTA(float, true);
     else TL_DELTA(float, false);
   } else {
-    if (dk % 4 == 0) TL_DELTA(bf16_t, true);
+    if (vec) TL_DELTA(bf16_t, true);
     else TL_DELTA(bf16_t, false);
   }
 #undef TL_DELTA

@@ -37,8 +37,10 @@ def paged_attention(
     n = qkv.shape[0]
     n_dec = ctx.host.n_decode
     v_dim = head_dim if v_head_dim is None else int(v_head_dim)
-    plain_only = softcap > 0 or chunk > 0 or sinks is not None or v_dim != head_dim
-    extras = dict(softcap=softcap, chunk=chunk, sinks=sinks, v_head_dim=v_dim) if plain_only else {}
+    plain_only = v_dim != head_dim  # (the MFMA kernels take a cap, chunks and sinks, but one head size)
+    extended = softcap > 0 or chunk > 0 or sinks is not None or plain_only
+    extras = dict(softcap=softcap, chunk=chunk, sinks=sinks, v_head_dim=v_dim) if extended else {}
+    fast_extras = dict(softcap=softcap, chunk=chunk, sinks=sinks) if extended else {}
     fast_decode = not plain_only and n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
     # the MFMA prefill kernel takes positive softmax scales only; anything else runs the plain kernel
     fast_prefill = (not plain_only and n_dec < n and scale > 0
@@ -54,11 +56,13 @@ def paged_attention(
             # the split-KV MFMA kernel
             if window > 0:
                 longest = min(longest, window + 15)
+            if chunk > 0:
+                longest = min(longest, chunk + 15)
             uneven = ctx.decode_uneven if ctx.decode_uneven is not None else ctx.host.decode_uneven
             ops.attention_decode(
                 qkv[:n_dec], n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.token_seq[:n_dec],
                 ctx.positions[:n_dec], ctx.block_tables[group], window, scale, longest, out=out[:n_dec],
-                uneven=uneven,
+                uneven=uneven, **fast_extras,
             )
         else:
             # the plain kernel: one wave a (token, head) would walk the whole context alone, so the
@@ -77,13 +81,15 @@ def paged_attention(
     if n_dec < n:
         if fast_prefill:
             qpt = ops.prefill_queries_per_tile(n_q_heads, n_kv_heads, head_dim)
-            key = ("prefill_tiles", qpt, window, n_kv_heads)
+            key = ("prefill_tiles", qpt, window, chunk, n_kv_heads)
             tiles = ctx.scratch.get(key)
             if tiles is None:
                 host = ctx.host
                 longest = int(max(host.kv_lens[n_dec : host.n_seqs]))
                 if window > 0:
                     longest = min(longest, window + qpt)
+                if chunk > 0:
+                    longest = min(longest, chunk + qpt)
                 key_groups = ops.prefill_key_groups(ops.prefill_tile_count(host.qo_indptr, n_dec, host.n_seqs, qpt), n_kv_heads, longest)
                 rows, q0s = ops.prefill_tiles(host.qo_indptr, n_dec, host.n_seqs, qpt, host.kv_lens, window)
                 both = torch.tensor([rows, q0s], dtype=torch.int32).to(qkv.device)
@@ -91,7 +97,7 @@ def paged_attention(
                 ctx.scratch[key] = tiles
             ops.attention_prefill(
                 qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, ctx.qo_indptr, ctx.kv_lens,
-                ctx.block_tables[group], tiles[0], tiles[1], window, scale, out, key_groups=tiles[2],
+                ctx.block_tables[group], tiles[0], tiles[1], window, scale, out, key_groups=tiles[2], **fast_extras,
             )
         else:
             ops.attention_generic(

@@ -137,7 +137,7 @@ def attention_generic_split(
 
 
 _DECODE_SIGNATURES = {
-    "tl_attn_decode": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _P],
+    "tl_attn_decode": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _F, _I, _P, _P],
 }
 DECODE_HEAD_DIMS = (32, 64, 128, 256)
 _DECODE_BLOCK_KEYS = 64  # keys one block pass covers (4 waves x 16): splits are multiples of it
@@ -218,10 +218,15 @@ def attention_decode(
     out: Optional[torch.Tensor] = None,
     split_size: Optional[int] = None,
     uneven: bool = False,
+    softcap: float = 0.0,
+    chunk: int = 0,
+    sinks: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Attention of single-token queries over their requests' pages with the split-KV MFMA kernel.
     ``longest``: an upper bound of any token's visible key range, counted from its 16-aligned first
-    visible key (position + 1 without a window)."""
+    visible key (position + 1 without a window).  ``softcap``, ``chunk``, ``sinks``: as ``attention_generic``."""
+    if sinks is not None and (not sinks.is_cuda or sinks.dtype != torch.float32 or sinks.numel() != n_q_heads or not sinks.is_contiguous()):
+        raise KernelError(f"attention_decode: sinks must be a contiguous float32 GPU vector of {n_q_heads} entries")
     _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
     _i32(token_seq, "token_seq")
     _i32(positions, "positions")
@@ -254,7 +259,7 @@ def attention_decode(
             qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
             token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
             n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), split_size, n_splits,
-            _ptr(ws_o), _ptr(ws_ml), _stream(),
+            _ptr(ws_o), _ptr(ws_ml), float(softcap), int(chunk), _ptr(sinks), _stream(),
         ),
         lib,
         "tl_variant_last_error",
@@ -264,7 +269,7 @@ def attention_decode(
 
 # ----------------------------------------------------------------------------- prefill attention (bfloat16, MFMA)
 _PREFILL_SIGNATURES = {
-    "tl_attn_prefill": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "tl_attn_prefill": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _I, _P, _P],
 }
 PREFILL_HEAD_DIMS = (32, 64, 128, 256)
 
@@ -359,6 +364,9 @@ def attention_prefill(
     scale: float,
     out: torch.Tensor,
     key_groups: int = 1,
+    softcap: float = 0.0,
+    chunk: int = 0,
+    sinks: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Causal attention of the rows named by the tile lists (see ``prefill_tiles``) with the MFMA
     prefill kernel.  Token t of ``qkv`` / ``out`` is token t of ``qo_indptr``'s numbering.
@@ -388,7 +396,7 @@ def attention_prefill(
             qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
             qo_indptr.data_ptr(), kv_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
             tile_row.data_ptr(), tile_q0.data_ptr(), tile_row.numel(), n_q_heads, n_kv_heads, head_dim, page_size,
-            window, float(scale), int(key_groups), _stream(),
+            window, float(scale), int(key_groups), float(softcap), int(chunk), _ptr(sinks), _stream(),
         ),
         lib,
         "tl_variant_last_error",
