@@ -201,7 +201,7 @@ rope_norm_kv_write_kernel(T* qkv, int row, int n_q, int n_kv, int dk, int dv, co
 // x: element (t, c) at x + t * x_stride + c, c < C (a slice of a projection's output).  Tokens of a
 // request are consecutive (qo_indptr); the request's K - 1 inputs before them are its history, 32-bit,
 // hist[k][c] at state + slot * state_stride + k * C + c, oldest first, zero for a new request.
-//   out[t, c] = act(bias[c] + sum_j taps[c][j] * in(t - (K - 1 - j))),  j ascending, 32-bit
+//   out[t, c] = act(bias[c] + sum_j taps[j][c] * in(t - (K - 1 - j))),  j ascending, 32-bit (taps: [K][C])
 // act 0: none, 1: silu.  The history is brought up to date by a second kernel, after every token has read it.
 template <typename T, int V>
 __global__ void __launch_bounds__(256)
@@ -233,7 +233,7 @@ causal_conv_kernel(const T* __restrict__ x, int x_stride, const float* __restric
       for (int e = 0; e < V; ++e) v[e] = hist[(size_t)(K - 1 + src) * C + c + e];
     }
 #pragma unroll
-    for (int e = 0; e < V; ++e) acc[e] = fmaf(taps[(size_t)(c + e) * K + j], v[e], acc[e]);
+    for (int e = 0; e < V; ++e) acc[e] = fmaf(taps[(size_t)j * C + c + e], v[e], acc[e]);
   }
   Vec o;
 #pragma unroll
@@ -286,7 +286,9 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
                       long long state_stride, const int32_t* __restrict__ qo_indptr, const int32_t* __restrict__ slot_ids,
                       T* __restrict__ out, int inner, int N, int lpc, const int32_t* __restrict__ segs,
                       float* __restrict__ seg_dt) {
-  extern __shared__ float bc_lds[];  // [kScanTile][2 * N]
+  extern __shared__ __attribute__((aligned(16))) float bc_lds[];  // [kScanTile][2 * N]
+  constexpr bool kFastExp = sizeof(T) == 2;
+  const bool vec4 = N % 4 == 0;
   const int row = blockIdx.y;  // (MODE 1, 2: the segment)
   const int start = MODE == 0 ? qo_indptr[row] : segs[2 * row], end = MODE == 0 ? qo_indptr[row + 1] : segs[2 * row + 1];
   const int per_block = kScanThreads / lpc;
@@ -302,6 +304,9 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
     const bool in = n0 + n < N;
     s[n] = in && MODE != 1 ? st[n0 + n] : 0.f;
     a[n] = in ? A[(size_t)c * N + n0 + n] : 0.f;
+    // with 16-bit activations the decay is one hardware exponential of a prescaled exponent (the kernel's time
+    // is its exponentials); with 32-bit ones the library's exp of the product as it is written
+    if (kFastExp) a[n] *= 1.4426950408889634f;
   }
   const float bias = dt_bias[c], dd = D[c];
   float dt_sum = 0.f;
@@ -318,10 +323,10 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
       if (MODE != 1) z_t[tt] = z[t * z_stride + c];
     }
     __syncthreads();  // everybody has finished with the tile before
-    for (int idx = threadIdx.x; idx < nt * 2 * N; idx += kScanThreads) {
-      const int tt = idx / (2 * N), e = idx % (2 * N);
+    for (int tt = 0; tt < nt; ++tt) {
       const T* src = bc + (size_t)(t0 + tt) * bc_stride;
-      bc_lds[idx] = to_f32(e < N ? src[b_off + e] : src[c_off + e - N]);
+      for (int e = threadIdx.x; e < 2 * N; e += kScanThreads)
+        bc_lds[tt * 2 * N + e] = to_f32(e < N ? src[b_off + e] : src[c_off + e - N]);
     }
     __syncthreads();
 #pragma unroll
@@ -336,11 +341,26 @@ selective_scan_kernel(const T* __restrict__ x, const DT* __restrict__ dt_pre, co
       const float* Bt = bc_lds + tt * 2 * N + n0;
       const float* Ct = Bt + N;
       float y = 0.f;
+      if (vec4) {  // N is a multiple of 4: four states' B and C a read (the same for every lane of a channel group)
 #pragma unroll
-      for (int n = 0; n < NB; ++n) {
-        if (n0 + n < N) {
-          s[n] = fmaf(expf(dt * a[n]), s[n], dx * Bt[n]);
-          y = fmaf(s[n], Ct[n], y);
+        for (int n = 0; n < NB; n += 4) {
+          if (n0 + n < N) {
+            const float4 b4 = *reinterpret_cast<const float4*>(Bt + n), c4 = *reinterpret_cast<const float4*>(Ct + n);
+            const float bb[4] = {b4.x, b4.y, b4.z, b4.w}, cc[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              s[n + e] = fmaf(kFastExp ? __builtin_amdgcn_exp2f(dt * a[n + e]) : expf(dt * a[n + e]), s[n + e], dx * bb[e]);
+              y = fmaf(s[n + e], cc[e], y);
+            }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+          if (n0 + n < N) {
+            s[n] = fmaf(kFastExp ? __builtin_amdgcn_exp2f(dt * a[n]) : expf(dt * a[n]), s[n], dx * Bt[n]);
+            y = fmaf(s[n], Ct[n], y);
+          }
         }
       }
       if (MODE != 1) {
@@ -399,8 +419,9 @@ scan_carry_kernel(float* __restrict__ ws, const float* __restrict__ seg_dt, cons
 // tile is worked on; in LDS the keys and queries are made unit vectors once per tile; then the tile's
 // tokens follow each other without a barrier (sums over a column's lanes by lane-to-lane moves).
 constexpr int kDeltaTile = 16;
-constexpr int kDeltaCols = 32;
-constexpr int kDeltaRows = 16;  // rows of a column that a lane holds
+// kDeltaCols, a template argument: 16 or 32 columns a block.  The time of a token is the block's multiply-adds, so
+// a launch of few blocks (a prompt of one request: heads * dv / 16 blocks, 256 for 32 heads of 128 columns) takes 16;
+// a launch that fills the GPU anyway (decode steps of many requests) takes 32 and has half the blocks to start.
 
 // Sum over groups of `width` neighbouring lanes (1, 2, 4, 8 or 16) by data-parallel moves inside a row
 // of 16 lanes: every lane of a group gets the same bits.
@@ -424,7 +445,9 @@ __device__ __forceinline__ float row_group_sum(float v, int width) {
   return v;
 }
 
-template <typename T, bool VEC>
+// kDeltaRows: rows of a column that a lane holds (8 for keys of up to 128 channels, else 16; a column's lanes lie
+// in one row of 16 lanes).
+template <typename T, bool VEC, int kDeltaRows, int kDeltaCols>
 __global__ void __launch_bounds__(512)
 gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int b_off,
                    int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
@@ -432,14 +455,14 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
                    const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int dk, int dv, int lpc,
                    int col_groups) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  // per token of the tile: k [dk], q [dk] (raw, then unit), v [kDeltaCols], o [kDeltaCols]; then beta, decay, 1/|k|, scale/|q|
+  // per token of the tile: k [dk], q [dk] (raw, then unit), v [kDeltaCols], o [kDeltaCols]; then six scalars
   const int dkp = dk + dk / 16 * 4;  // a token's keys in LDS: four floats of padding after every sixteen, so that
                                      // the lanes of a column, sixteen rows apart, read different banks
   float* k_l = lds;
   float* q_l = k_l + kDeltaTile * dkp;
   float* v_l = q_l + kDeltaTile * dkp;
   float* o_l = v_l + kDeltaTile * kDeltaCols;
-  float* sc_l = o_l + kDeltaTile * kDeltaCols;  // [kDeltaTile][4]
+  float* sc_l = o_l + kDeltaTile * kDeltaCols;  // [kDeltaTile][6]: beta, decay, 1/|k|, scale/|q|, k^ . q^
   const int row = blockIdx.y;
   const int h = blockIdx.x / col_groups, cg = blockIdx.x % col_groups;
   const int g = h / (H / G);
@@ -469,7 +492,12 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
 
   // what a thread fetches of a tile: element e of the tile's keys and queries (e = tt * 2 dk + d, d < dk a
   // key's channel, else a query's) for e = tid, tid + threads, ...; likewise of the values
-  constexpr int kPreKQ = 16, kPreV = 8;
+  // (element e = tt * 2 dk + d of a tile without a division: from one pass to the next a thread's element moves on
+  // by the block's threads, which are less than two tokens' worth)
+  const int two_dk = 2 * dk;
+  const int tt_first = threadIdx.x / two_dk, d_first = threadIdx.x % two_dk;
+  const int tt_step = n_threads / two_dk, d_step = n_threads % two_dk;
+  constexpr int kPreKQ = kDeltaRows == 16 && kDeltaCols == 16 ? 32 : 16, kPreV = 8;  // (a tile's elements over the block's threads, at most)
   T pre_kq[kPreKQ], pre_v[kPreV], pre_b = from_f32<T>(0.f), pre_a = from_f32<T>(0.f);
   auto fetch = [&](int t0) {
     const int nt = min(kDeltaTile, end - t0);
@@ -478,11 +506,13 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
       pre_b = pr[b_off + h];
       pre_a = pr[a_off + h];
     }
+    int tt = tt_first, d = d_first;
 #pragma unroll
     for (int u = 0; u < kPreKQ; ++u) {
-      const int e = threadIdx.x + u * n_threads;
-      const int tt = e / (2 * dk), d = e % (2 * dk);
       if (tt < nt) pre_kq[u] = qkv[(size_t)(t0 + tt) * qkv_stride + (d < dk ? k_col + d : q_col + d - dk)];
+      tt += tt_step;
+      d += d_step;
+      if (d >= two_dk) { d -= two_dk; ++tt; }
     }
 #pragma unroll
     for (int u = 0; u < kPreV; ++u) {
@@ -495,12 +525,16 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
   for (int t0 = start; t0 < end; t0 += kDeltaTile) {
     const int nt = min(kDeltaTile, end - t0);
     __syncthreads();  // the tile before has been read to its end
+    {
+      int tt = tt_first, d = d_first;
 #pragma unroll
-    for (int u = 0; u < kPreKQ; ++u) {
-      const int e = threadIdx.x + u * n_threads;
-      const int tt = e / (2 * dk), d = e % (2 * dk);
-      const int dd = d < dk ? d : d - dk;
-      if (tt < nt) (d < dk ? k_l : q_l)[tt * dkp + dd + dd / 16 * 4] = to_f32(pre_kq[u]);
+      for (int u = 0; u < kPreKQ; ++u) {
+        const int dd = d < dk ? d : d - dk;
+        if (tt < nt) (d < dk ? k_l : q_l)[tt * dkp + dd + dd / 16 * 4] = to_f32(pre_kq[u]);
+        tt += tt_step;
+        d += d_step;
+        if (d >= two_dk) { d -= two_dk; ++tt; }
+      }
     }
 #pragma unroll
     for (int u = 0; u < kPreV; ++u) {
@@ -509,76 +543,111 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
       if (tt < nt && d < v_cols) v_l[tt * kDeltaCols + d] = to_f32(pre_v[u]);
     }
     if (threadIdx.x < nt) {
-      sc_l[4 * threadIdx.x] = sigmoid_f(to_f32(pre_b));
-      sc_l[4 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pre_a) + bias));
+      sc_l[6 * threadIdx.x] = sigmoid_f(to_f32(pre_b));
+      sc_l[6 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pre_a) + bias));
     }
     if (t0 + kDeltaTile < end) fetch(t0 + kDeltaTile);  // on its way while this tile is worked on
     __syncthreads();
-    // the norms: 2 nt vectors, each summed by eight neighbouring lanes (a lane its channels in ascending
-    // order, the lanes by moves in a fixed order); every thread of the first waves takes part in the moves
-    for (int v0 = 0; v0 < 2 * kDeltaTile; v0 += n_threads / 8) {
-      const int vec = v0 + threadIdx.x / 8, sub = threadIdx.x % 8;
-      const int tt = vec / 2, which = vec % 2;
-      float ss = 0.f;
+    // per token the sums of squares of its key and its query and their product, each by eight neighbouring
+    // lanes (a lane its channels in ascending order, the lanes by moves in a fixed order)
+    for (int v0 = 0; v0 < kDeltaTile; v0 += n_threads / 8) {
+      const int tt = v0 + threadIdx.x / 8, sub = threadIdx.x % 8;
+      float kk2 = 0.f, qq2 = 0.f, kq = 0.f;
       if (tt < nt) {
-        const float* src = (which ? q_l : k_l) + tt * dkp;
         for (int d = sub; d < dk; d += 8) {
-          const float e = src[d + d / 16 * 4];
-          ss = fmaf(e, e, ss);
+          const float ke = k_l[tt * dkp + d + d / 16 * 4], qe = q_l[tt * dkp + d + d / 16 * 4];
+          kk2 = fmaf(ke, ke, kk2);
+          qq2 = fmaf(qe, qe, qq2);
+          kq = fmaf(ke, qe, kq);
         }
       }
-      ss = row_group_sum(ss, 8);
-      if (tt < nt && sub == 0) sc_l[4 * tt + 2 + which] = (which ? q_scale : 1.0f) / sqrtf(ss + 1e-6f);
+      kk2 = row_group_sum(kk2, 8);
+      qq2 = row_group_sum(qq2, 8);
+      kq = row_group_sum(kq, 8);
+      if (tt < nt && sub == 0) {
+        const float k_inv = 1.0f / sqrtf(kk2 + 1e-6f), q_inv = q_scale / sqrtf(qq2 + 1e-6f);
+        sc_l[6 * tt + 2] = k_inv;
+        sc_l[6 * tt + 3] = q_inv;
+        sc_l[6 * tt + 4] = kq * k_inv * q_inv;  // k^ . q^
+      }
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < nt * 2 * dk; e += n_threads) {
-      const int tt = e / (2 * dk), d = e % (2 * dk);
-      const int dd = d < dk ? d : d - dk;
-      (d < dk ? k_l : q_l)[tt * dkp + dd + dd / 16 * 4] *= sc_l[4 * tt + (d < dk ? 2 : 3)];
+    {  // every thread scales the elements that it put there
+      int tt = tt_first, d = d_first;
+#pragma unroll
+      for (int u = 0; u < kPreKQ; ++u) {
+        const int dd = d < dk ? d : d - dk;
+        if (tt < nt) (d < dk ? k_l : q_l)[tt * dkp + dd + dd / 16 * 4] *= sc_l[6 * tt + (d < dk ? 2 : 3)];
+        tt += tt_step;
+        d += d_step;
+        if (d >= two_dk) { d -= two_dk; ++tt; }
+      }
     }
     __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const float beta = sc_l[4 * tt], decay = sc_l[4 * tt + 1];
+    // One token: S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  The read-out follows from the
+    // decayed state and u, o = (decay S)^T q + u (k . q), so both products with the state are taken in one walk
+    // over the lane's rows and summed over the column's lanes together, and the state's update is no part of
+    // the chain that o waits for.  A token's operands are read from LDS while the token before is worked on.
+    struct Operands {
+      float kk[kDeltaRows], qq[kDeltaRows], v, beta, decay, kq;
+    };
+    auto read = [&](Operands& x, int tt_raw) {
+      const int tt = tt_raw < kDeltaTile ? tt_raw : kDeltaTile - 1;
       const float* kt = k_l + tt * dkp + i0 + i0 / 16 * 4;  // (i0 is a multiple of 16: a lane's rows have no padding between them)
       const float* qt = q_l + tt * dkp + i0 + i0 / 16 * 4;
-      float kk[kDeltaRows], qq[kDeltaRows];
       if (VEC) {  // dk is a multiple of 4: four channels a read
 #pragma unroll
         for (int r = 0; r < kDeltaRows; r += 4) {
           const bool in = i0 + r < dk;
           const float4 k4 = in ? *reinterpret_cast<const float4*>(kt + r) : float4{0.f, 0.f, 0.f, 0.f};
           const float4 q4 = in ? *reinterpret_cast<const float4*>(qt + r) : float4{0.f, 0.f, 0.f, 0.f};
-          kk[r] = k4.x; kk[r + 1] = k4.y; kk[r + 2] = k4.z; kk[r + 3] = k4.w;
-          qq[r] = q4.x; qq[r + 1] = q4.y; qq[r + 2] = q4.z; qq[r + 3] = q4.w;
+          x.kk[r] = k4.x; x.kk[r + 1] = k4.y; x.kk[r + 2] = k4.z; x.kk[r + 3] = k4.w;
+          x.qq[r] = q4.x; x.qq[r + 1] = q4.y; x.qq[r + 2] = q4.z; x.qq[r + 3] = q4.w;
         }
       } else {
 #pragma unroll
         for (int r = 0; r < kDeltaRows; ++r) {
-          kk[r] = i0 + r < dk ? kt[r] : 0.f;
-          qq[r] = i0 + r < dk ? qt[r] : 0.f;
+          x.kk[r] = i0 + r < dk ? kt[r] : 0.f;
+          x.qq[r] = i0 + r < dk ? qt[r] : 0.f;
         }
       }
-      float kv[4] = {0.f, 0.f, 0.f, 0.f};
+      x.v = v_l[tt * kDeltaCols + (j_loc < kDeltaCols ? j_loc : 0)];
+      x.beta = sc_l[6 * tt];
+      x.decay = sc_l[6 * tt + 1];
+      x.kq = sc_l[6 * tt + 4];
+    };
+    auto token = [&](const Operands& x, int tt) {
+      float kv[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < kDeltaRows; ++r) {
-        S[r] = decay * S[r];
-        kv[r % 4] = fmaf(S[r], kk[r], kv[r % 4]);
+        S[r] = x.decay * S[r];
+        kv[r % 4] = fmaf(S[r], x.kk[r], kv[r % 4]);
+        sq[r % 4] = fmaf(S[r], x.qq[r], sq[r % 4]);
       }
-      const float kv_all = row_group_sum((kv[0] + kv[1]) + (kv[2] + kv[3]), lpc);
-      const float u = beta * (v_l[tt * kDeltaCols + (j_loc < kDeltaCols ? j_loc : 0)] - kv_all);
-      float o[4] = {0.f, 0.f, 0.f, 0.f};
+      float kv_all = (kv[0] + kv[1]) + (kv[2] + kv[3]), sq_all = (sq[0] + sq[1]) + (sq[2] + sq[3]);
+      if (lpc >= 2) { kv_all += dpp_xor1(kv_all); sq_all += dpp_xor1(sq_all); }
+      if (lpc >= 4) { kv_all += dpp_xor2(kv_all); sq_all += dpp_xor2(sq_all); }
+      if (lpc >= 8) { kv_all += dpp_half_mirror(kv_all); sq_all += dpp_half_mirror(sq_all); }
+      if (lpc >= 16) { kv_all += dpp_mirror(kv_all); sq_all += dpp_mirror(sq_all); }
+      const float u = x.beta * (x.v - kv_all);
+      if (live && part == 0) o_l[tt * kDeltaCols + j_loc] = fmaf(u, x.kq, sq_all);
 #pragma unroll
-      for (int r = 0; r < kDeltaRows; ++r) {
-        S[r] = fmaf(kk[r], u, S[r]);
-        o[r % 4] = fmaf(S[r], qq[r], o[r % 4]);
+      for (int r = 0; r < kDeltaRows; ++r) S[r] = fmaf(x.kk[r], u, S[r]);
+    };
+    Operands xa, xb;
+    read(xa, 0);
+    for (int tt = 0; tt < nt; tt += 2) {
+      read(xb, tt + 1);
+      token(xa, tt);
+      if (tt + 1 < nt) {
+        read(xa, tt + 2);
+        token(xb, tt + 1);
       }
-      const float o_all = row_group_sum((o[0] + o[1]) + (o[2] + o[3]), lpc);
-      if (live && part == 0) o_l[tt * kDeltaCols + j_loc] = o_all;
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < nt * v_cols; e += n_threads) {
-      const int tt = e / v_cols, d = e % v_cols;
-      o_raw[((size_t)(t0 + tt) * H + h) * dv + cg * kDeltaCols + d] = o_l[tt * kDeltaCols + d];
+    for (int e = threadIdx.x; e < nt * kDeltaCols; e += n_threads) {
+      const int tt = e / kDeltaCols, d = e % kDeltaCols;
+      if (d < v_cols) o_raw[((size_t)(t0 + tt) * H + h) * dv + cg * kDeltaCols + d] = o_l[tt * kDeltaCols + d];
     }
   }
   if (live) {
@@ -798,16 +867,26 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
   TL_REQUIRE(o_raw != nullptr, "gated_delta: no workspace");
   if (n_seqs == 0 || n_tokens == 0) return TL_OK;
   if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "gated_delta: unknown dtype %d", dtype);
+  const int rows = dk <= 128 ? 8 : 16;
   int lpc = 1;
-  while (kDeltaRows * lpc < dk) lpc *= 2;  // at most 16: a column's lanes lie in one row of 16 lanes
-  const int threads = (kDeltaCols * lpc + kWave - 1) / kWave * kWave;
-  const int col_groups = (dv + kDeltaCols - 1) / kDeltaCols;
-  const size_t lds = ((size_t)kDeltaTile * (2 * (dk + dk / 16 * 4) + 2 * kDeltaCols + 4)) * sizeof(float);
+  while (rows * lpc < dk) lpc *= 2;  // at most 16: a column's lanes lie in one row of 16 lanes
+  // columns a block: 16 while that leaves fewer than two blocks a CU, else 32
+  const int cols = (long long)n_seqs * H * ((dv + 15) / 16) < 2LL * tl_device_facts().compute_units ? 16 : 32;
+  const int threads = (cols * lpc + kWave - 1) / kWave * kWave;
+  const int col_groups = (dv + cols - 1) / cols;
+  const size_t lds = ((size_t)kDeltaTile * (2 * (dk + dk / 16 * 4) + 2 * cols + 6)) * sizeof(float);
   const dim3 grid(H * col_groups, n_seqs);
-#define TL_DELTA(T, VEC)                                                                                               \
-  gated_delta_kernel<T, VEC><<<grid, threads, lds, stream>>>((const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, \
-                                                             a_off, A_log, dt_bias, state, state_stride, qo_indptr, slot_ids, \
-                                                             o_raw, H, G, dk, dv, lpc, col_groups)
+#define TL_DELTA_R(T, VEC, R, C)                                                                                       \
+  gated_delta_kernel<T, VEC, R, C><<<grid, threads, lds, stream>>>((const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, \
+                                                                   a_off, A_log, dt_bias, state, state_stride, qo_indptr, slot_ids, \
+                                                                   o_raw, H, G, dk, dv, lpc, col_groups)
+#define TL_DELTA(T, VEC)                                \
+  do {                                                  \
+    if (rows == 8 && cols == 16) TL_DELTA_R(T, VEC, 8, 16);   \
+    else if (rows == 8) TL_DELTA_R(T, VEC, 8, 32);      \
+    else if (cols == 16) TL_DELTA_R(T, VEC, 16, 16);    \
+    else TL_DELTA_R(T, VEC, 16, 32);                    \
+  } while (0)
   // four rows a load where every lane's rows start at a multiple of 16 bytes, in LDS and in the state
   const bool vec = dk % 4 == 0 && ((uintptr_t)state % 16) == 0 && state_stride % 4 == 0;
   if (dtype == TL_F32) {
@@ -818,6 +897,7 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
     else TL_DELTA(bf16_t, false);
   }
 #undef TL_DELTA
+#undef TL_DELTA_R
   int rc = tl_check_launch("gated_delta");
   if (rc != TL_OK) return rc;
   for (int t0 = 0; t0 < n_tokens; t0 += 65535) {

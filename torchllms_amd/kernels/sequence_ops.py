@@ -179,16 +179,16 @@ def causal_conv(
     silu: bool = True,
 ) -> torch.Tensor:
     """Causal convolution over time, channel by channel, of ``x`` [n, C] (a view of some columns of a
-    matrix will do) with ``taps`` float32 [C, K] (the last column multiplies the current token) and
+    matrix will do) with ``taps`` float32 [K, C] (the last row multiplies the current token) and
     ``bias`` float32 [C] or None, then silu.  What lies before a request's first token of this step is
     its history: (K - 1) * C floats at ``state_offset`` of its state row, which is brought up to date."""
     _gpu(x, taps, bias)
     if x.dim() != 2 or x.stride(1) != 1:
         raise KernelError("causal_conv: x must be a matrix whose rows are contiguous")
     n, C = x.shape
-    if taps.dim() != 2 or taps.shape[0] != C or taps.dtype != torch.float32 or not taps.is_contiguous():
-        raise KernelError(f"causal_conv: taps must be contiguous float32 [{C}, K]")
-    K = taps.shape[1]
+    if taps.dim() != 2 or taps.shape[1] != C or taps.dtype != torch.float32 or not taps.is_contiguous():
+        raise KernelError(f"causal_conv: taps must be contiguous float32 [K, {C}]")
+    K = taps.shape[0]
     if bias is not None and (bias.shape != (C,) or bias.dtype != torch.float32 or not bias.is_contiguous()):
         raise KernelError(f"causal_conv: bias must be a float32 vector of {C} entries")
     n_seqs = _step_rows(token_seq, qo_indptr, slot_ids, n, state)

@@ -61,7 +61,7 @@ class SelectiveScan(Mixer):
         self.w_x = tensors["x"].contiguous()
         self.w_dt = tensors["dt"].contiguous()
         self.w_o = tensors["o"].contiguous()
-        self.conv_w = tensors["conv"].float().contiguous()
+        self.conv_w = tensors["conv"].float().t().contiguous()  # [taps, channels]: a tap's weights lie side by side
         self.conv_b = tensors["conv.b"].float().contiguous()
         self.dt_b = tensors["dt.b"].float().contiguous()
         self.A = (-torch.exp(tensors["A_log"].float())).contiguous()
@@ -139,7 +139,7 @@ class GatedDelta(Mixer):
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         # one projection [q | k | v | output gate | write strength | decay]: a single product per step
         self.w_all = torch.cat([tensors[n] for n in ("q", "k", "v", "g", "b", "a")], dim=0).contiguous()
-        self.conv_w = torch.cat([tensors[n + ".conv"] for n in ("q", "k", "v")], dim=0).float().contiguous()
+        self.conv_w = torch.cat([tensors[n + ".conv"] for n in ("q", "k", "v")], dim=0).float().t().contiguous()  # [taps, channels]
         self.w_o = tensors["o"].contiguous()
         self.A_log = tensors["A_log"].float().contiguous()
         self.dt_bias = tensors["dt_bias"].float().contiguous()
