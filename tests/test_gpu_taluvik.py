@@ -128,6 +128,8 @@ ALONE = {
     "delta_odd": models.layer("delta", {"heads": 3, "kv_heads": 1, "dim": 18, "vdim": 70, "conv": 3}),
     "mamba1": models.layer("mamba1", {"inner": 72, "state": 24, "dt_rank": 6, "conv": 3}),
     "mamba1_many_states": models.layer("mamba1", {"inner": 40, "state": 100, "dt_rank": 8, "conv": 6}),
+    # a step-size rank that the decode products for 17 to 128 rows take (K a multiple of 128), read as a view of columns
+    "mamba1_wide_rank": models.layer("mamba1", {"inner": 64, "state": 16, "dt_rank": 128, "conv": 4}),
     "feed_forward": models.layer("mamba1", {"inner": 8, "state": 1, "dt_rank": 1, "conv": 1}, ff=136),
 }
 
@@ -352,6 +354,38 @@ def test_greedy_generation_through_the_entry_point(tmp_path):
     for p, r in zip(prompts, llm16.generate(prompt_token_ids=prompts, temperature=0.0, max_new_tokens=4)):
         logits = plain.forward(cfg, w64, p)[-1]
         assert logits[r.token_ids[0]] >= logits.max() - 0.05 * float(logits.std())
+
+
+def test_generate_command_line_with_random_weights(tmp_path):
+    """The generate program given nothing but a config.json: ``--random-weights --seed`` draws the weights that
+    ``write_model_folder`` would write for that seed, so the plain model can say which tokens to expect."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from torchllms_amd.config import TaluvikConfig
+    from torchllms_amd.weights import write_model_folder
+
+    root = Path(__file__).resolve().parent.parent
+    folder = tmp_path / "only_config"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(models.CONFIGS["B"]))
+    prompt = random_tokens(13, models.CONFIGS["B"]["vocab"], 21)
+    proc = subprocess.run(
+        [sys.executable, "-m", "torchllms_amd.inference.generate", "--model", str(folder), "--dtype", "float32", "--random-weights",
+         "--seed", "7", "--max-new-tokens", "6", "--prompt-ids", *map(str, prompt)],
+        capture_output=True, text=True, cwd=root, timeout=300,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [int(t) for t in proc.stdout.split()[-6:]]
+    written = write_model_folder(tmp_path / "written", TaluvikConfig.from_dict(models.CONFIGS["B"]), seed=7, dtype=torch.float32)
+    cfg, weights = models.read_folder(written)
+    w64 = {k: v.double() for k, v in weights.items()}
+    toks = list(prompt)
+    for _ in range(6):
+        toks.append(int(plain.forward(cfg, w64, toks)[-1].argmax()))
+    assert got == toks[len(prompt):]
 
 
 def test_trace_replay_program(tmp_path):

@@ -55,7 +55,14 @@ __device__ __forceinline__ short4_t hi_half(u32x4_t v) { return __builtin_bit_ca
 enum Epilogue { kPlain = 0, kGated = 1, kQkv = 2, kGatedHalf = 3, kResidual = 4 };
 
 // What the variants need that stand in for a norm.
+// The gate's activation: 0 silu, 1 gelu in its tanh form.
+__device__ __forceinline__ float gate_activation(float g, int act) {
+  if (act == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.0f + expf(-g));
+}
+
 struct NormArgs {
+  int act;  // kGated, kGatedHalf: the gate's activation (see gate_activation)
   // kGated, kGatedHalf, kQkv: the rows of A are to be read as A[m] / sqrt(sum[m] / width + eps);
   // row_sums [n_row_sums][16] are pieces of sum[m] (piece by piece, the 16 rows side by side).  Null: A as it is.
   const float* row_sums;
@@ -332,7 +339,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
         if (n >= N) continue;
         const float g = to_f32(from_f32<OutT>(acc[0][i]));
         const float u = to_f32(from_f32<OutT>(up[i]));
-        const float act = to_f32(from_f32<OutT>(g / (1.0f + expf(-g))));
+        const float act = to_f32(from_f32<OutT>(gate_activation(g, na.act)));
         C[(size_t)n16 * ldc + n] = from_f32<OutT>(act * u);
       }
     }
@@ -369,7 +376,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
       if constexpr (GLU) {
         const float g = to_f32(from_f32<OutT>(acc[0][i]));
         const float u = to_f32(from_f32<OutT>(acc[1][i]));
-        const float act = to_f32(from_f32<OutT>(g / (1.0f + expf(-g))));
+        const float act = to_f32(from_f32<OutT>(gate_activation(g, na.act)));
         C[(size_t)n16 * ldc + n] = from_f32<OutT>(act * u);
       } else {
         C[(size_t)n16 * ldc + n] = from_f32<OutT>(acc[0][i]);
@@ -473,15 +480,17 @@ TL_EXPORT int tl_gemm_stream(const void* A, int lda, const void* W, int ldw, voi
 }
 
 // The gated pair of products: W [2 N, K] = gate rows | up rows; C [M, N] bfloat16 =
-// silu(A gate^T) * (A up^T), rounded as the two products, the activation and the final product
-// would be if each were stored in bfloat16.  cols: 16 or 8 columns of C per block.
+// act(A gate^T) * (A up^T), act = silu (0) or the tanh form of gelu (1), rounded as the two products, the
+// activation and the final product would be if each were stored in bfloat16.  cols: 16 or 8 columns of C per block.
 // row_sums [n_row_sums][16] 32-bit or null: pieces of a sum of squares per row, as tl_gemm_stream_residual
 // leaves them; then row m of both products is scaled by 1 / sqrt(sum / K + eps) before the roundings.
 TL_EXPORT int tl_gemm_stream_glu(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N,
                                  int K, int waves, int cols, const float* row_sums, int n_row_sums, float eps,
-                                 hipStream_t stream) {
+                                 int act, hipStream_t stream) {
   TL_REQUIRE(cols == 8 || cols == 16, "gemm_stream_glu: cols must be 8 or 16");
+  TL_REQUIRE(act == 0 || act == 1, "gemm_stream_glu: activation %d (0: silu, 1: gelu_tanh)", act);
   NormArgs na = {};
+  na.act = act;
   na.row_sums = row_sums; na.n_row_sums = n_row_sums; na.width = (float)K; na.eps = eps;
   return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, cols == 8 ? kGatedHalf : kGated, QkvArgs{}, na, stream);
 }

@@ -241,6 +241,42 @@ causal_conv_kernel(const T* __restrict__ x, int x_stride, const float* __restric
   *reinterpret_cast<Vec*>(out + (size_t)t * out_stride + c) = o;
 }
 
+// A step in which every request brings one token (decode): convolution and new history in one kernel.  A thread
+// owns V channels of one request: it reads their history, adds the token, and writes the history back one place on.
+template <typename T, int V>
+__global__ void __launch_bounds__(256)
+conv_step_kernel(const T* __restrict__ x, int x_stride, const float* __restrict__ taps, const float* __restrict__ bias,
+                 float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
+                 const int32_t* __restrict__ slot_ids, T* __restrict__ out, int out_stride, int C, int K, int act) {
+  const int c = (blockIdx.x * blockDim.x + threadIdx.x) * V;
+  if (c >= C) return;
+  const int row = blockIdx.y;
+  const int t = qo_indptr[row];
+  float* hist = state + (long long)slot_ids[row] * state_stride;
+  struct alignas(sizeof(T) * V) Vec { T e[V]; };
+  const Vec in = *reinterpret_cast<const Vec*>(x + (size_t)t * x_stride + c);
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = bias ? bias[c + e] : 0.f;
+  for (int j = 0; j < K - 1; ++j) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float v = hist[(size_t)j * C + c + e];
+      acc[e] = fmaf(taps[(size_t)j * C + c + e], v, acc[e]);
+      if (j > 0) hist[(size_t)(j - 1) * C + c + e] = v;  // (entry j - 1 has been read in the pass before)
+    }
+  }
+  Vec o;
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const float v = to_f32(in.e[e]);
+    acc[e] = fmaf(taps[(size_t)(K - 1) * C + c + e], v, acc[e]);
+    if (K > 1) hist[(size_t)(K - 2) * C + c + e] = v;
+    o.e[e] = from_f32<T>(act == 1 ? silu_f(acc[e]) : acc[e]);
+  }
+  *reinterpret_cast<Vec*>(out + (size_t)t * out_stride + c) = o;
+}
+
 // New history of every request of the step: the last K - 1 entries of (old history, the step's inputs).
 template <typename T>
 __global__ void __launch_bounds__(256)
@@ -448,6 +484,8 @@ __device__ __forceinline__ float row_group_sum(float v, int width) {
 // kDeltaRows: rows of a column that a lane holds (8 for keys of up to 128 channels, else 16; a column's lanes lie
 // in one row of 16 lanes).
 template <typename T, bool VEC, int kDeltaRows, int kDeltaCols>
+// (Held to 128 registers, so that more of a decode step's many short blocks share a CU, the compiler spills 400 to
+// 1,000 bytes a lane: what the tile's pipeline carries is more than that.  It is left its 233 to 256.)
 __global__ void __launch_bounds__(512)
 gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int b_off,
                    int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
@@ -636,6 +674,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
     };
     Operands xa, xb;
     read(xa, 0);
+#pragma unroll 1
     for (int tt = 0; tt < nt; tt += 2) {
       read(xb, tt + 1);
       token(xa, tt);
@@ -763,6 +802,21 @@ TL_EXPORT int tl_causal_conv(const void* x, int x_stride, const float* taps, con
   const int elt = dtype == TL_F32 ? 4 : 2, vec = 16 / elt;
   const bool wide = C % vec == 0 && x_stride % vec == 0 && out_stride % vec == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)out % 16) == 0;
   const int vblocks = (C / (wide ? vec : 1) + 255) / 256;
+  if (n_tokens == n_seqs) {  // one token a request: convolution and history in one launch
+    const dim3 grid(vblocks, n_seqs);
+#define TL_CONV_STEP(T, V)                                                                                            \
+  conv_step_kernel<T, V><<<grid, 256, 0, stream>>>((const T*)x, x_stride, taps, bias, state, state_stride, qo_indptr, \
+                                                   slot_ids, (T*)out, out_stride, C, K, act)
+    if (dtype == TL_F32) {
+      if (wide) TL_CONV_STEP(float, 4);
+      else TL_CONV_STEP(float, 1);
+    } else {
+      if (wide) TL_CONV_STEP(bf16_t, 8);
+      else TL_CONV_STEP(bf16_t, 1);
+    }
+#undef TL_CONV_STEP
+    return tl_check_launch("conv_step");
+  }
   for (int t0 = 0; t0 < n_tokens; t0 += 65535) {
     const int nt = n_tokens - t0 < 65535 ? n_tokens - t0 : 65535;
     const dim3 grid(vblocks, nt);

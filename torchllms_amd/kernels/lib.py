@@ -43,7 +43,7 @@ _CORE_SIGNATURES = {
     "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
     "tl_gemm_f32": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
-    "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _P],
+    "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _I, _P],
     "tl_gemm_stream_residual": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _P, _I, _F, _P],
     "tl_gemm_wide": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P],

@@ -279,11 +279,18 @@ def gemm_wide_qkv(
     return out
 
 
-def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0, cols: int = 16, norm: Optional[NormedRows] = None) -> torch.Tensor:
-    """``silu(x @ gate.T) * (x @ up.T)`` for at most 16 rows of bfloat16 ``x`` and ``w`` [2F, K] =
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0, cols: int = 16, norm: Optional[NormedRows] = None,
+                    activation: str = "silu") -> torch.Tensor:
+    """``act(x @ gate.T) * (x @ up.T)`` for at most 16 rows of bfloat16 ``x`` and ``w`` [2F, K] =
     gate rows | up rows, in one pass over ``w``; rounded as ``silu_mul(linear(x, w))``.  ``cols``: 16
     or 8 columns of the result per block (8: a launch shaped like the plain product's).  ``norm``:
-    ``NormedRows`` whose ``gained`` rows ``x`` is; the result is then that of the normed rows."""
+    ``NormedRows`` whose ``gained`` rows ``x`` is; the result is then that of the normed rows.
+    ``activation``: "silu" or "gelu_tanh"."""
+    if activation not in GATE_ACTIVATIONS:
+        raise KernelError(f"gemm_stream_glu: activation {activation!r} ({sorted(GATE_ACTIVATIONS)})")
     _gpu(x, w)
     sums, n_sums, eps = _norm_args(norm, x)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
@@ -296,7 +303,7 @@ def gemm_stream_glu(x: torch.Tensor, w: torch.Tensor, waves: int = 0, cols: int 
     check(
         core().tl_gemm_stream_glu(
             x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k, waves, cols, sums, n_sums, eps,
-            _stream(),
+            GATE_ACTIVATIONS[activation], _stream(),
         )
     )
     return out
@@ -641,13 +648,21 @@ def linear_glu(x: torch.Tensor, w: torch.Tensor, activation: str = "silu") -> to
     """``act(x @ gate.T) * (x @ up.T)`` for ``w`` [2F, K] = gate rows | up rows.  With silu: one fused
     kernel where one of the decode kernels serves the shape, else the product followed by the gate.  ``x``
     may be ``NormedRows``: the weight-streaming kernel applies them, for any other they are normed first.
-    With "gelu_tanh" the product is followed by the gate's kernel."""
+    With "gelu_tanh" the weight-streaming kernel (up to 16 rows) takes the gate into itself as well; every other
+    product is followed by the gate's kernel."""
     if activation != "silu":
         if activation != "gelu_tanh":
             raise KernelError(f"linear_glu: activation {activation!r} (silu, gelu_tanh)")
         from .sequence_ops import gelu_mul
 
-        return gelu_mul(linear(resolved(x), w))
+        x = resolved(x)
+        if x.dtype == torch.bfloat16:
+            _gpu(x, w)
+            choice = linear_choice(x, w, "glu")
+            if choice is not None and choice[0] == "stream":
+                return gemm_stream_glu(x, w, choice[1], choice[2] if len(choice) > 2 else 16, activation=activation)
+            return gelu_mul(run_choice(choice, x, w, x.dtype))
+        return gelu_mul(linear(x, w))
     if isinstance(x, NormedRows):
         choice = linear_choice(x.gained, w, "glu")
         if choice is not None and choice[0] == "stream":

@@ -37,8 +37,7 @@ class SwiGLU(FeedForward):
         self.w2 = tensors["w2.weight"].contiguous()
 
     def linear_weights(self):
-        # (only the silu gate has fused forms; another activation runs the plain product and then the gate)
-        return [(self.w13, "glu" if self.activation == "silu" else "plain"), (self.w2, "sum")]
+        return [(self.w13, "glu"), (self.w2, "sum")]
 
     def forward(self, x, ctx):
         return ops.linear_to_sum(ops.linear_glu(x, self.w13, self.activation), self.w2, may_wait=True)
