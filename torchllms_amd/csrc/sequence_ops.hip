@@ -135,6 +135,8 @@ int gelu_mul_launch(const T* gate_up, T* out, int n, int inter, hipStream_t stre
 constexpr int kHeadWaves = 4;
 constexpr int kHeadChan = 4;  // channels a lane holds: heads of up to 256
 
+constexpr int kHeadsPerWave = 2;  // heads a wave takes, all their loads asked for before anything waits for one
+
 template <typename T>
 __global__ void __launch_bounds__(kHeadWaves* kWave)
 rope_norm_kv_write_kernel(T* qkv, int row, int n_q, int n_kv, int dk, int dv, const float2* __restrict__ cos_sin,
@@ -142,58 +144,76 @@ rope_norm_kv_write_kernel(T* qkv, int row, int n_q, int n_kv, int dk, int dv, co
                           const int32_t* __restrict__ slot_mapping, int page_size) {
   const int t = blockIdx.x;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int unit = blockIdx.y * kHeadWaves + wave;
-  if (unit >= n_q + 2 * n_kv) return;
+  const int unit0 = (blockIdx.y * kHeadWaves + wave) * kHeadsPerWave;
+  const int n_units = n_q + 2 * n_kv;
+  if (unit0 >= n_units) return;
   T* base = qkv + (size_t)t * row;
   const int slot = slot_mapping ? slot_mapping[t] : -1;
   const bool store = k_pages != nullptr && slot >= 0;
   const size_t page = store ? slot / page_size : 0;
   const int off = store ? slot % page_size : 0;
-  if (unit >= n_q + n_kv) {  // a value head: copied
-    if (!store || v_pages == nullptr) return;
-    const int kh = unit - n_q - n_kv;
-    const T* src = base + (size_t)(n_q + n_kv) * dk + (size_t)kh * dv;
-    T* dst = v_pages + ((page * n_kv + kh) * page_size + off) * dv;
-    for (int d = lane; d < dv; d += kWave) dst[d] = src[d];
-    return;
-  }
-  T* head = base + (size_t)unit * dk;
   const int rh = rot / 2;
-  float val[kHeadChan];
-  float ss = 0.f;
+  // a unit is a query head, a key head or a value head (copied); units past the last do nothing
+  float val[kHeadsPerWave][kHeadChan];
+  float ss[kHeadsPerWave];
 #pragma unroll
-  for (int c = 0; c < kHeadChan; ++c) {
-    const int d = lane + c * kWave;
-    val[c] = 0.f;
-    if (d < dk) {
-      const float a = to_f32(head[d]);
-      float v = a;
-      if (d < rot) {
-        int i, partner;
-        bool first;
-        if (pairing == 0) {
-          i = d / 2; first = (d % 2) == 0; partner = first ? d + 1 : d - 1;
-        } else {
-          first = d < rh; i = first ? d : d - rh; partner = first ? d + rh : d - rh;
+  for (int u = 0; u < kHeadsPerWave; ++u) {
+    const int unit = unit0 + u;
+    ss[u] = 0.f;
+    const bool rotated = unit < n_q + n_kv;
+    const bool value = !rotated && unit < n_units;
+    const T* head = rotated ? base + (size_t)unit * dk : base + (size_t)(n_q + n_kv) * dk + (size_t)(value ? unit - n_q - n_kv : 0) * dv;
+    const int width = rotated ? dk : dv;
+#pragma unroll
+    for (int c = 0; c < kHeadChan; ++c) {
+      const int d = lane + c * kWave;
+      val[u][c] = 0.f;
+      if ((rotated || value) && d < width) {
+        const float a = to_f32(head[d]);
+        float v = a;
+        if (rotated && d < rot) {
+          int i, partner;
+          bool first;
+          if (pairing == 0) {
+            i = d / 2; first = (d % 2) == 0; partner = first ? d + 1 : d - 1;
+          } else {
+            first = d < rh; i = first ? d : d - rh; partner = first ? d + rh : d - rh;
+          }
+          const float o = to_f32(head[partner]);
+          const float2 cs = cos_sin[(size_t)t * rh + i];
+          v = first ? a * cs.x - o * cs.y : a * cs.x + o * cs.y;
         }
-        const float o = to_f32(head[partner]);
-        const float2 cs = cos_sin[(size_t)t * rh + i];
-        v = first ? a * cs.x - o * cs.y : a * cs.x + o * cs.y;
+        val[u][c] = v;
+        ss[u] += v * v;
       }
-      val[c] = v;
-      ss += v * v;
     }
   }
-  ss = wave_sum(ss);  // (every load of the head lies before this exchange, every store behind it)
-  const float inv = norm_eps > 0.f ? 1.0f / sqrtf(ss / (float)dk + norm_eps) : 1.0f;
-  const bool is_q = unit < n_q;
-  T* dst = head;
-  if (!is_q && store) dst = k_pages + ((page * n_kv + (unit - n_q)) * page_size + off) * dk;
-  if (!is_q && k_pages != nullptr && !store) return;  // a token without a slot keeps nothing
 #pragma unroll
-  for (int c = 0; c < kHeadChan; ++c) {
-    const int d = lane + c * kWave;
-    if (d < dk) dst[d] = from_f32<T>(val[c] * inv);
+  for (int u = 0; u < kHeadsPerWave; ++u) ss[u] = wave_sum(ss[u]);  // (every load lies before these exchanges, every store behind)
+#pragma unroll
+  for (int u = 0; u < kHeadsPerWave; ++u) {
+    const int unit = unit0 + u;
+    if (unit >= n_units) continue;
+    if (unit >= n_q + n_kv) {  // a value head: copied into its page
+      if (!store || v_pages == nullptr) continue;
+      T* dst = v_pages + ((page * n_kv + (unit - n_q - n_kv)) * page_size + off) * dv;
+#pragma unroll
+      for (int c = 0; c < kHeadChan; ++c) {
+        const int d = lane + c * kWave;
+        if (d < dv) dst[d] = from_f32<T>(val[u][c]);
+      }
+      continue;
+    }
+    const float inv = norm_eps > 0.f ? 1.0f / sqrtf(ss[u] / (float)dk + norm_eps) : 1.0f;
+    const bool is_q = unit < n_q;
+    if (!is_q && k_pages != nullptr && !store) continue;  // a token without a slot keeps nothing
+    T* dst = base + (size_t)unit * dk;
+    if (!is_q && store) dst = k_pages + ((page * n_kv + (unit - n_q)) * page_size + off) * dk;
+#pragma unroll
+    for (int c = 0; c < kHeadChan; ++c) {
+      const int d = lane + c * kWave;
+      if (d < dk) dst[d] = from_f32<T>(val[u][c] * inv);
+    }
   }
 }
 
@@ -767,14 +787,15 @@ TL_EXPORT int tl_rope_norm_kv_write(void* qkv, int n_tokens, int n_q, int n_kv, 
                                     int pairing, float norm_eps, void* k_pages, void* v_pages, const int32_t* slot_mapping,
                                     int page_size, int dtype, hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q > 0 && n_kv >= 0 && dk > 0 && dv > 0, "rope_norm: bad sizes");
-  TL_REQUIRE(dk <= kHeadChan * kWave, "rope_norm: heads of %d channels, at most %d", dk, kHeadChan * kWave);
+  TL_REQUIRE(dk <= kHeadChan * kWave && dv <= kHeadChan * kWave, "rope_norm: heads of %d and %d channels, at most %d", dk, dv, kHeadChan * kWave);
   TL_REQUIRE(rot >= 0 && rot <= dk && rot % 2 == 0, "rope_norm: %d rotated channels of %d (even, at most the head)", rot, dk);
   TL_REQUIRE(pairing == 0 || pairing == 1, "rope_norm: pairing must be 0 (interleaved) or 1 (half split)");
   TL_REQUIRE(rot == 0 || cos_sin != nullptr, "rope_norm: rotation without a table of cosines and sines");
   TL_REQUIRE(k_pages == nullptr || (v_pages != nullptr && slot_mapping != nullptr && page_size > 0), "rope_norm: pages without slots");
   if (n_tokens == 0) return TL_OK;
   const int row = (n_q + n_kv) * dk + n_kv * dv;
-  const dim3 grid(n_tokens, (n_q + 2 * n_kv + kHeadWaves - 1) / kHeadWaves);
+  const int per_block = kHeadWaves * kHeadsPerWave;
+  const dim3 grid(n_tokens, (n_q + 2 * n_kv + per_block - 1) / per_block);
   if (dtype == TL_F32)
     rope_norm_kv_write_kernel<float><<<grid, kHeadWaves * kWave, 0, stream>>>(
         (float*)qkv, row, n_q, n_kv, dk, dv, (const float2*)cos_sin, rot, pairing, norm_eps, (float*)k_pages, (float*)v_pages,
