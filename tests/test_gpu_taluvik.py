@@ -531,3 +531,59 @@ def test_random_configurations(tmp_path, seed):
             assert sum(seen) / len(seen) < BF16_TOL, f"mean distance {sum(seen) / len(seen)}  {cfg_dict}"
             assert sum(d > 2 * BF16_TOL for d in seen) <= len(seen) // 50, f"{sum(d > 2 * BF16_TOL for d in seen)} of {len(seen)} positions  {cfg_dict}"
         del engine
+
+
+# ----------------------------------------------------------------------------- sizes of the order of a real model's layers
+LARGER = {
+    "architecture": "Taluvik", "vocab": 1000, "width": 1024, "embedding": {"scale": 4.0}, "norm": {"eps": 1e-5},
+    "residual_mult": 0.5,
+    "layers": [
+        models.layer("mamba1", {"inner": 2048, "state": 16, "dt_rank": 64, "conv": 4}, ff=2816),
+        models.layer("attention", models.attention(16, 4, 128, 128, 64, 256, 0.09, 30.0, base=500000.0,
+                                                   scaling={"factor": 8.0, "low": 1.0, "high": 4.0, "original": 128}), ff=2816),
+        models.layer("delta", {"heads": 8, "kv_heads": 4, "dim": 128, "vdim": 128, "conv": 4}, ff=2816),
+        models.layer("attention", models.attention(16, 16, 64, 64, 64, 100, 0.125, 20.0), ff=2816),
+    ],
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layers_of_larger_sizes(tmp_path, dtype):
+    """Heads of 128 and 64 that the matrix-core attention kernels take, a delta rule of 128 by 128 (eight rows a lane,
+    sixteen lanes a column, 16 and 32 columns a block), a scan over 2,048 channels in segments, products that the
+    library, the streaming kernel and the kernel for 17 to 128 rows serve: a prompt of 700 tokens whole, then a
+    second request in portions beside single tokens of the first, then sixteen requests decoding together."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    folder = models.make_folder(tmp_path / "m", LARGER, seed=21)
+    cfg, weights = models.read_folder(folder)
+    requests = {"a": random_tokens(740, cfg["vocab"], 1), "b": random_tokens(300, cfg["vocab"], 2)}
+    requests.update({f"d{i}": random_tokens(40 + 3 * i, cfg["vocab"], 10 + i) for i in range(16)})
+    truth, scale = truth_of(cfg, weights, requests)
+    tol = FP32_TOL if dtype == "float32" else BF16_TOL
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=160, max_seqs=18)
+    worst = 0.0
+
+    def step(entries):
+        nonlocal worst
+        logits = engine.step(entries).cpu()
+        k = 0
+        for e in entries:
+            base = engine.num_tokens(e.rid) - len(e.tokens)
+            for w in e.want:
+                worst = max(worst, distance(logits[k], truth[e.rid][base + w], scale))
+                k += 1
+
+    for rid in requests:
+        engine.admit(rid)
+    step([StepEntry("a", requests["a"][:700], list(range(0, 700, 7)) + [699])])
+    at = 0
+    for n in (130, 2, 64, 1, 33, 70):
+        step([StepEntry("b", requests["b"][at : at + n], list(range(n))), StepEntry("a", [requests["a"][700 + at // 50]], [0])]
+             if at < 250 and engine.num_tokens("a") == 700 + at // 50 else [StepEntry("b", requests["b"][at : at + n], list(range(n)))])
+        at += n
+    assert at == 300
+    step([StepEntry(f"d{i}", requests[f"d{i}"][:-8], [len(requests[f"d{i}"]) - 9]) for i in range(16)])
+    for j in range(8, 0, -1):
+        step([StepEntry(f"d{i}", [requests[f"d{i}"][-j]], [0]) for i in range(16)])
+    assert worst < tol, worst

@@ -278,12 +278,25 @@ conv_step_kernel(const T* __restrict__ x, int x_stride, const float* __restrict_
   float acc[V];
 #pragma unroll
   for (int e = 0; e < V; ++e) acc[e] = bias ? bias[c + e] : 0.f;
-  for (int j = 0; j < K - 1; ++j) {
+  // eight entries of the history are asked for at once (a store between two loads of the same array makes the
+  // second wait for the first); entry j moves to place j - 1, which has been read before
+  constexpr int kAhead = 8;
+  for (int j0 = 0; j0 < K - 1; j0 += kAhead) {
+    float hv[kAhead][V];
 #pragma unroll
-    for (int e = 0; e < V; ++e) {
-      const float v = hist[(size_t)j * C + c + e];
-      acc[e] = fmaf(taps[(size_t)j * C + c + e], v, acc[e]);
-      if (j > 0) hist[(size_t)(j - 1) * C + c + e] = v;  // (entry j - 1 has been read in the pass before)
+    for (int u = 0; u < kAhead; ++u)
+#pragma unroll
+      for (int e = 0; e < V; ++e) hv[u][e] = j0 + u < K - 1 ? hist[(size_t)(j0 + u) * C + c + e] : 0.f;
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int j = j0 + u;
+      if (j < K - 1) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          acc[e] = fmaf(taps[(size_t)j * C + c + e], hv[u][e], acc[e]);
+          if (j > 0) hist[(size_t)(j - 1) * C + c + e] = hv[u][e];
+        }
+      }
     }
   }
   Vec o;
@@ -722,6 +735,97 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
   }
 }
 
+// The same recurrence for a step in which every request brings one token (decode): no tiles, nothing fetched
+// ahead, few registers, so that many of these short blocks share a CU.  Every sum is taken in the order in which
+// gated_delta_kernel takes it (the norms by eight lanes over every eighth channel, the products with the state by
+// four chains a lane and then the column's lanes), so a token's result has the same bits from either kernel.
+template <typename T, bool VEC, int kDeltaRows>
+__global__ void __launch_bounds__(512)
+gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int b_off,
+                        int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+                        float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
+                        const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int dk, int dv,
+                        int lpc, int col_groups) {
+  constexpr int kCols = 32;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int dkp = dk + dk / 16 * 4;
+  float* k_l = lds;
+  float* q_l = lds + dkp;
+  const int row = blockIdx.y;
+  const int h = blockIdx.x / col_groups, cg = blockIdx.x % col_groups;
+  const int g = h / (H / G);
+  const size_t t = (size_t)qo_indptr[row];
+  const int j_loc = threadIdx.x / lpc, part = threadIdx.x % lpc;
+  const int j_raw = cg * kCols + j_loc;
+  const bool live = j_loc < kCols && j_raw < dv;
+  const int j = j_raw < dv ? j_raw : dv - 1;
+  const int i0 = part * kDeltaRows;
+  const T* tok = qkv + t * qkv_stride;
+  for (int d = threadIdx.x; d < 2 * dk; d += blockDim.x) {
+    const int dd = d < dk ? d : d - dk;
+    (d < dk ? k_l : q_l)[dd + dd / 16 * 4] = to_f32(tok[d < dk ? G * dk + g * dk + dd : g * dk + dd]);
+  }
+  float* st = state + (long long)slot_ids[row] * state_stride + ((size_t)h * dv + j) * dk;
+  float S[kDeltaRows];
+  if (VEC) {
+#pragma unroll
+    for (int r = 0; r < kDeltaRows; r += 4) {
+      const float4 s4 = i0 + r < dk ? *reinterpret_cast<const float4*>(st + i0 + r) : float4{0.f, 0.f, 0.f, 0.f};
+      S[r] = s4.x; S[r + 1] = s4.y; S[r + 2] = s4.z; S[r + 3] = s4.w;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < kDeltaRows; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
+  }
+  const float v = to_f32(tok[2 * G * dk + h * dv + j]);
+  const float pb = to_f32(proj[t * proj_stride + b_off + h]), pa = to_f32(proj[t * proj_stride + a_off + h]);
+  const float neg_rate = -expf(A_log[h]), bias = dt_bias[h];
+  __syncthreads();
+  const int sub = threadIdx.x % 8;
+  float kk2 = 0.f, qq2 = 0.f, kq = 0.f;
+  for (int d = sub; d < dk; d += 8) {
+    const float ke = k_l[d + d / 16 * 4], qe = q_l[d + d / 16 * 4];
+    kk2 = fmaf(ke, ke, kk2);
+    qq2 = fmaf(qe, qe, qq2);
+    kq = fmaf(ke, qe, kq);
+  }
+  kk2 = row_group_sum(kk2, 8);
+  qq2 = row_group_sum(qq2, 8);
+  kq = row_group_sum(kq, 8);
+  const float k_inv = 1.0f / sqrtf(kk2 + 1e-6f), q_inv = (1.0f / sqrtf((float)dk)) / sqrtf(qq2 + 1e-6f);
+  const float kq_hat = kq * k_inv * q_inv;
+  const float beta = sigmoid_f(pb), decay = expf(neg_rate * softplus_f(pa + bias));
+  float kv[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
+  float kk[kDeltaRows];
+#pragma unroll
+  for (int r = 0; r < kDeltaRows; ++r) {
+    const int i = i0 + r;
+    const bool in = i < dk;
+    kk[r] = in ? k_l[i + i / 16 * 4] * k_inv : 0.f;
+    const float qq = in ? q_l[i + i / 16 * 4] * q_inv : 0.f;
+    S[r] = decay * S[r];
+    kv[r % 4] = fmaf(S[r], kk[r], kv[r % 4]);
+    sq[r % 4] = fmaf(S[r], qq, sq[r % 4]);
+  }
+  const float kv_all = row_group_sum((kv[0] + kv[1]) + (kv[2] + kv[3]), lpc);
+  const float sq_all = row_group_sum((sq[0] + sq[1]) + (sq[2] + sq[3]), lpc);
+  const float u = beta * (v - kv_all);
+  if (live && part == 0) o_raw[(t * H + h) * dv + j] = fmaf(u, kq_hat, sq_all);
+#pragma unroll
+  for (int r = 0; r < kDeltaRows; ++r) S[r] = fmaf(kk[r], u, S[r]);
+  if (live) {
+    if (VEC) {
+#pragma unroll
+      for (int r = 0; r < kDeltaRows; r += 4)
+        if (i0 + r < dk) *reinterpret_cast<float4*>(st + i0 + r) = float4{S[r], S[r + 1], S[r + 2], S[r + 3]};
+    } else {
+#pragma unroll
+      for (int r = 0; r < kDeltaRows; ++r)
+        if (i0 + r < dk) st[i0 + r] = S[r];
+    }
+  }
+}
+
 // out[t, h, :] = T(o / sqrt(mean(o^2) + eps) * norm_w * silu(gate[t, h, :])): one wave a (token, head).
 template <typename T>
 __global__ void __launch_bounds__(kHeadWaves* kWave)
@@ -945,8 +1049,9 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
   const int rows = dk <= 128 ? 8 : 16;
   int lpc = 1;
   while (rows * lpc < dk) lpc *= 2;  // at most 16: a column's lanes lie in one row of 16 lanes
-  // columns a block: 16 while that leaves fewer than two blocks a CU, else 32
-  const int cols = (long long)n_seqs * H * ((dv + 15) / 16) < 2LL * tl_device_facts().compute_units ? 16 : 32;
+  // columns a block: 16 while that leaves fewer than two blocks a CU, else 32 (a step of single tokens: always 32)
+  const bool single = n_tokens == n_seqs;
+  const int cols = !single && (long long)n_seqs * H * ((dv + 15) / 16) < 2LL * tl_device_facts().compute_units ? 16 : 32;
   const int threads = (cols * lpc + kWave - 1) / kWave * kWave;
   const int col_groups = (dv + cols - 1) / cols;
   const size_t lds = ((size_t)kDeltaTile * (2 * (dk + dk / 16 * 4) + 2 * cols + 6)) * sizeof(float);
@@ -964,13 +1069,34 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
   } while (0)
   // four rows a load where every lane's rows start at a multiple of 16 bytes, in LDS and in the state
   const bool vec = dk % 4 == 0 && ((uintptr_t)state % 16) == 0 && state_stride % 4 == 0;
-  if (dtype == TL_F32) {
+#define TL_DELTA_STEP(T, VEC)                                                                                          \
+  do {                                                                                                                 \
+    const size_t step_lds = 2 * (size_t)(dk + dk / 16 * 4) * sizeof(float);                                            \
+    if (rows == 8)                                                                                                     \
+      gated_delta_step_kernel<T, VEC, 8><<<grid, threads, step_lds, stream>>>(                                         \
+          (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,   \
+          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups);                                                  \
+    else                                                                                                               \
+      gated_delta_step_kernel<T, VEC, 16><<<grid, threads, step_lds, stream>>>(                                        \
+          (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,   \
+          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups);                                                  \
+  } while (0)
+  if (single) {
+    if (dtype == TL_F32) {
+      if (vec) TL_DELTA_STEP(float, true);
+      else TL_DELTA_STEP(float, false);
+    } else {
+      if (vec) TL_DELTA_STEP(bf16_t, true);
+      else TL_DELTA_STEP(bf16_t, false);
+    }
+  } else if (dtype == TL_F32) {
     if (vec) TL_DELTA(float, true);
     else TL_DELTA(float, false);
   } else {
     if (vec) TL_DELTA(bf16_t, true);
     else TL_DELTA(bf16_t, false);
   }
+#undef TL_DELTA_STEP
 #undef TL_DELTA
 #undef TL_DELTA_R
   int rc = tl_check_launch("gated_delta");
