@@ -123,6 +123,8 @@ ALONE = {
     # cap low enough to bend most scores
     "attention_matrix_cores_64": models.layer("attention", models.attention(8, 2, 64, 64, 32, 48, 0.6, 4.0)),
     "attention_matrix_cores_128": models.layer("attention", models.attention(4, 1, 128, 128, 64, 100, 0.4, 5.0, base=300.0)),
+    "attention_matrix_cores_256": models.layer("attention", models.attention(2, 1, 256, 256, 128, 70, 0.05, 12.0)),
+    "attention_matrix_cores_32": models.layer("attention", models.attention(16, 1, 32, 32, 32, 64, 0.7, 8.0)),
     "delta": models.layer("delta", {"heads": 4, "kv_heads": 2, "dim": 24, "vdim": 40, "conv": 4}),
     "delta_wide": models.layer("delta", {"heads": 1, "kv_heads": 1, "dim": 256, "vdim": 64, "conv": 2}),
     "delta_odd": models.layer("delta", {"heads": 3, "kv_heads": 1, "dim": 18, "vdim": 70, "conv": 3}),
@@ -145,7 +147,8 @@ def test_a_mechanism_alone(tmp_path, what, dtype):
     cfg, weights = models.read_folder(folder)
     tokens = random_tokens(275, cfg["vocab"], 9)
     truth, scale = truth_of(cfg, weights, {"r": tokens})
-    engine = Engine.from_folder(folder, dtype=dtype, page_size=8, num_pages=80, max_seqs=2)
+    page = 16 if what.endswith("_32") else 8  # (the matrix-core prefill kernel wants 512 / head size tokens a page)
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=page, num_pages=640 // page, max_seqs=2)
     engine.admit("whole")
     whole = engine.step([StepEntry("whole", tokens, list(range(len(tokens))))]).cpu()
     engine.admit("cut")
@@ -587,3 +590,42 @@ def test_layers_of_larger_sizes(tmp_path, dtype):
     for j in range(8, 0, -1):
         step([StepEntry(f"d{i}", [requests[f"d{i}"][-j]], [0]) for i in range(16)])
     assert worst < tol, worst
+
+
+@pytest.mark.parametrize("head_dim", [32, 64, 128, 256])
+def test_matrix_core_attention_agrees_with_the_plain_kernel(head_dim):
+    """The split-KV decode kernel and the tiled prefill kernel with a cap, chunks and sinks against the plain
+    kernel on the same pages and queries: a prompt portion behind cached keys beside two single tokens, chunks
+    that end inside the portion and inside a tile of keys."""
+    from torchllms_amd.engine.context import upload
+    from torchllms_amd.engine.layout import StepEntry, build_step_layout
+    from torchllms_amd.kernels import ops
+    from torchllms_amd.kernels.attention import paged_attention
+
+    dev = "cuda:0"
+    G = 2
+    H = G * (4 if head_dim < 256 else 2)
+    page, chunk = 16, 88
+    entries = [StepEntry("p", [0] * 150, []), StepEntry("d", [0], []), StepEntry("e", [0], [])]
+    starts = [70, 200, 87]
+    tables = [[list(range(0, 14)), list(range(14, 27)), list(range(27, 33))]]
+    layout = build_step_layout(entries, starts, [0, 1, 2], tables, [page])
+    assert layout.n_decode == 2
+    ctx = upload(layout, dev)
+    g = torch.Generator().manual_seed(head_dim)
+    qkv = torch.randn((152, H * head_dim), generator=g).to(torch.bfloat16).to(dev)
+    k_pages = torch.randn((40, G, page, head_dim), generator=g).to(torch.bfloat16).to(dev)
+    v_pages = torch.randn((40, G, page, head_dim), generator=g).to(torch.bfloat16).to(dev)
+    extras = dict(softcap=6.0, chunk=chunk, sinks=torch.randn(H, generator=g).to(dev))
+    scale = 2.5 / head_dim ** 0.5
+    assert ops.decode_attention_supported(torch.bfloat16, H, G, head_dim)
+    assert ops.prefill_attention_supported(torch.bfloat16, H, G, head_dim, page)
+    fast = paged_attention(qkv, H, G, head_dim, k_pages, v_pages, ctx, 0, 0, scale, **extras).float()
+    plain_out = ops.attention_generic(qkv, H, G, head_dim, k_pages, v_pages, ctx.token_seq, ctx.positions, ctx.block_tables[0],
+                                      0, scale, v_head_dim=head_dim, **extras).float()
+    assert (fast - plain_out).abs().max() < 0.03, (fast - plain_out).abs().max()
+    # what the comparison would miss if both forgot the same thing: the plain kernel alone notices each of the three
+    for change in (dict(extras, softcap=0.0), dict(extras, chunk=0), dict(extras, sinks=None)):
+        other = ops.attention_generic(qkv, H, G, head_dim, k_pages, v_pages, ctx.token_seq, ctx.positions, ctx.block_tables[0],
+                                      0, scale, v_head_dim=head_dim, **change).float()
+        assert (other - plain_out).abs().max() > 0.1
