@@ -47,10 +47,16 @@ class CacheGroupSpec:
     page_size: int = 0  # tokens per page; 0: the manager's default
     dtype: Optional[str] = None  # "float32" / "bfloat16"; None: the manager's default
     v_head_dim: int = 0  # head size of the values; 0: that of the keys
+    values_in_keys: bool = False  # a token's value is the first channels of its key row: no value pages
 
     @property
     def value_dim(self) -> int:
         return self.v_head_dim or self.head_dim
+
+    @property
+    def elements_per_token(self) -> int:
+        """Cached elements of one token in one layer of the group."""
+        return self.num_kv_heads * (self.head_dim + (0 if self.values_in_keys else self.value_dim))
 
 
 @dataclass(frozen=True)
@@ -75,7 +81,7 @@ def group_layers(needs: Sequence[Tuple[Hashable, object]]) -> Tuple[List[CacheGr
         if hasattr(need, "num_kv_heads"):
             v_dim = int(getattr(need, "v_head_dim", None) or 0)
             form = (need.num_kv_heads, need.head_dim, need.window, int(getattr(need, "page_size", None) or 0),
-                    getattr(need, "dtype", None), 0 if v_dim == need.head_dim else v_dim)
+                    getattr(need, "dtype", None), 0 if v_dim == need.head_dim else v_dim, bool(getattr(need, "values_in_keys", False)))
             kv.setdefault(form, []).append(run_id)
         elif hasattr(need, "shape"):
             st.setdefault((tuple(need.shape), need.dtype), []).append(run_id)
@@ -83,8 +89,8 @@ def group_layers(needs: Sequence[Tuple[Hashable, object]]) -> Tuple[List[CacheGr
             raise TypeError(f"cache entry {run_id}: unknown cache need {need!r}")
     groups = [
         CacheGroupSpec(name=f"kv{i}", run_ids=tuple(runs), num_kv_heads=h, head_dim=d, window=w, page_size=p, dtype=t,
-                       v_head_dim=vd)
-        for i, ((h, d, w, p, t, vd), runs) in enumerate(kv.items())
+                       v_head_dim=vd, values_in_keys=vk)
+        for i, ((h, d, w, p, t, vd, vk), runs) in enumerate(kv.items())
     ]
     states = [
         StateSlotSpec(name=f"state{i}", run_ids=tuple(runs), shape=shape, dtype=dtype)
@@ -220,7 +226,9 @@ class CacheManager:
             for gi, (g, pool) in enumerate(zip(self.groups, self.pools)):
                 shape = (len(g.run_ids), pool.num_pages, g.num_kv_heads, self.page_sizes[gi])
                 self.k_pages.append(torch.zeros(shape + (g.head_dim,), dtype=self.dtypes[gi], device=device))
-                self.v_pages.append(torch.zeros(shape + (g.value_dim,), dtype=self.dtypes[gi], device=device))
+                # (values that live inside the key rows: the mixer's value pages are its key pages)
+                self.v_pages.append(self.k_pages[-1] if g.values_in_keys else
+                                    torch.zeros(shape + (g.value_dim,), dtype=self.dtypes[gi], device=device))
             for s in self.states:
                 shape = (len(s.run_ids), max_seqs, *s.shape)
                 self.state_tensors.append(torch.zeros(shape, dtype=getattr(torch, s.dtype), device=device))
@@ -233,7 +241,7 @@ class CacheManager:
         total = 0
         for g in groups:
             elt = torch.empty(0, dtype=getattr(torch, g.dtype) if g.dtype else dtype).element_size()
-            total += len(g.run_ids) * g.num_kv_heads * (g.head_dim + g.value_dim) * elt
+            total += len(g.run_ids) * g.elements_per_token * elt
         return total
 
     @staticmethod
@@ -459,7 +467,7 @@ class CacheManager:
         page_size = self.page_sizes[gi]
         n = e.num_tokens
         k = torch.zeros((n, g.num_kv_heads, g.head_dim), dtype=self.dtypes[gi], device=self.device)
-        v = torch.zeros((n, g.num_kv_heads, g.value_dim), dtype=self.dtypes[gi], device=self.device)
+        v = torch.zeros((n, g.num_kv_heads, g.head_dim if g.values_in_keys else g.value_dim), dtype=self.dtypes[gi], device=self.device)
         for b, page in enumerate(e.block_tables[gi]):
             lo = b * page_size
             hi = min(lo + page_size, n)

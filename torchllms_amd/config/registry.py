@@ -17,6 +17,7 @@ from typing import Any, Callable, Dict, List, Optional, Sequence
 from .llama import ConfigError, LlamaConfig, llama_model_spec
 from .spec import ModelSpec
 from .taluvik import ARCHITECTURE as TALUVIK, TaluvikConfig, taluvik_model_spec
+from .vobolorn import ARCHITECTURE as VOBOLORN, VobolornConfig, vobolorn_model_spec
 
 
 @dataclass(frozen=True)
@@ -161,5 +162,28 @@ register_architecture(
         weight_rules=_taluvik_rules,
         stop_token_ids=_taluvik_stop_ids,
         config_type=TaluvikConfig,
+    )
+)
+
+
+def _vobolorn_rules(cfg: VobolornConfig):
+    from ..weights.names import vobolorn_name_rules
+
+    return vobolorn_name_rules(cfg)
+
+
+def _vobolorn_stop_ids(cfg: VobolornConfig):
+    eos = cfg.eos_token_id
+    return [] if eos is None else (list(eos) if isinstance(eos, (list, tuple)) else [eos])
+
+
+register_architecture(
+    ArchSpec(
+        name=VOBOLORN,
+        config_from_dict=VobolornConfig.from_dict,
+        model_spec=vobolorn_model_spec,
+        weight_rules=_vobolorn_rules,
+        stop_token_ids=_vobolorn_stop_ids,
+        config_type=VobolornConfig,
     )
 )

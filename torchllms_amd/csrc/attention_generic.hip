@@ -14,7 +14,8 @@
 namespace {
 
 constexpr int kWavesPerBlock = 4;
-constexpr int kMaxHeadDim = 256;
+constexpr int kMaxHeadDim = 256;   // of the values: a lane adds up kMaxHeadDim / 64 channels of the output
+constexpr int kMaxKeyDim = 512;    // of queries and keys, which only enter the scores
 constexpr int kChanPerLane = kMaxHeadDim / kWave;
 constexpr int kTileMinTokens = 32;  // steps with at least this many tokens share keys and values through LDS
 
@@ -50,7 +51,7 @@ struct Query {
   const T* k_pages;
   const T* v_pages;
   const int32_t* bt;        // the request's block table
-  int n_kv_heads, g, head_dim, v_dim, page_size;
+  int n_kv_heads, g, head_dim, v_dim, v_pitch, page_size;  // v_pitch: elements between two value rows
   int lo, p;                // the keys it sees: positions lo .. p
   float scale, softcap;
 };
@@ -132,7 +133,7 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int src = jj + u <= jj_hi ? jj + u : jj_hi;  // rows past the end: fetched again, never added
-      const T* vr = a.v_pages + __shfl(row_at, src, kWave) * a.v_dim;
+      const T* vr = a.v_pages + __shfl(row_at, src, kWave) * a.v_pitch;
       pw[u] = __shfl(pj, src, kWave);
 #pragma unroll
       for (int c = 0; c < kChanPerLane; ++c) {
@@ -171,11 +172,11 @@ __device__ __forceinline__ Query<T> make_query(const float* qs, const T* k_pages
                                                const int32_t* token_seq, const int32_t* positions,
                                                const int32_t* block_table, int bt_stride, int t, int h, int n_q_heads,
                                                int n_kv_heads, int head_dim, int page_size, int window, float scale,
-                                               float softcap, int chunk, int v_dim) {
+                                               float softcap, int chunk, int v_dim, int v_pitch) {
   Query<T> a;
   a.qs = qs; a.k_pages = k_pages; a.v_pages = v_pages;
   a.bt = block_table + (size_t)token_seq[t] * bt_stride;
-  a.n_kv_heads = n_kv_heads; a.g = h / (n_q_heads / n_kv_heads); a.head_dim = head_dim; a.v_dim = v_dim;
+  a.n_kv_heads = n_kv_heads; a.g = h / (n_q_heads / n_kv_heads); a.head_dim = head_dim; a.v_dim = v_dim; a.v_pitch = v_pitch;
   a.page_size = page_size;
   a.p = positions[t];
   a.lo = first_key(a.p, window, chunk);
@@ -192,8 +193,8 @@ attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
                          const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ block_table, int bt_stride, int n_q_heads,
                          int n_kv_heads, int head_dim, int page_size, int window, float scale, float softcap,
-                         int chunk, const float* __restrict__ sinks, int v_dim) {
-  __shared__ float q_lds[kWavesPerBlock][kMaxHeadDim];
+                         int chunk, const float* __restrict__ sinks, int v_dim, int v_pitch) {
+  __shared__ float q_lds[kWavesPerBlock][kMaxKeyDim];
   const int t = blockIdx.x;
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
@@ -204,7 +205,7 @@ attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave][d] = to_f32(qv[d]);
   __syncthreads();
   const Query<T> a = make_query<T>(q_lds[wave], k_pages, v_pages, token_seq, positions, block_table, bt_stride, t, h,
-                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim);
+                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim, v_pitch);
   float acc[kChanPerLane];
 #pragma unroll
   for (int c = 0; c < kChanPerLane; ++c) acc[c] = 0.f;
@@ -302,7 +303,7 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
                       const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                       const int32_t* __restrict__ block_table, int bt_stride, int n_tokens, int n_q_heads,
                       int n_kv_heads, int head_dim, int page_size, int window, float scale, int heads_per_block,
-                      float softcap, int chunk, const float* __restrict__ sinks, int v_dim) {
+                      float softcap, int chunk, const float* __restrict__ sinks, int v_dim, int v_pitch) {
   extern __shared__ __attribute__((aligned(16))) float tile_lds[];
   const int pitch = head_dim + kTilePad, pitch_v = v_dim + kTilePad;
   float* q_lds = tile_lds;                          // [kTileWaves][head_dim]
@@ -322,7 +323,7 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave * head_dim + d] = to_f32(qv[d]);
   const Query<T> a = make_query<T>(q_lds + wave * head_dim, k_pages, v_pages, token_seq, positions, block_table,
                                    bt_stride, t, h, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap,
-                                   chunk, v_dim);
+                                   chunk, v_dim, v_pitch);
   // what the whole block sees: the same for every thread, from the tokens' own entries
   const int last = min(t0 + QT, n_tokens) - 1;
   const int seq0 = token_seq[t0];
@@ -366,7 +367,7 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
         const size_t row_at = ((size_t)page * n_kv_heads + g) * page_size + (size_t)(j % page_size);
         const bool is_k = piece_kv < per_k;
         const int piece = is_k ? piece_kv : piece_kv - per_k;
-        const T* src = is_k ? k_pages + row_at * head_dim : v_pages + row_at * v_dim;
+        const T* src = is_k ? k_pages + row_at * head_dim : v_pages + row_at * v_pitch;
         float* dst = is_k ? k_t + r * pitch : v_t + r * pitch_v;
         if (VEC) {
           float e[4];
@@ -408,8 +409,8 @@ attention_blocks_kernel(const T* __restrict__ q, int q_stride, const T* __restri
                         const T* __restrict__ v_pages, const int32_t* __restrict__ token_seq,
                         const int32_t* __restrict__ positions, const int32_t* __restrict__ block_table, int bt_stride,
                         int n_q_heads, int n_kv_heads, int head_dim, int page_size, int window, float scale,
-                        float* __restrict__ partials, int max_blocks, float softcap, int chunk, int v_dim) {
-  __shared__ float q_lds[kWavesPerBlock][kMaxHeadDim];
+                        float* __restrict__ partials, int max_blocks, float softcap, int chunk, int v_dim, int v_pitch) {
+  __shared__ float q_lds[kWavesPerBlock][kMaxKeyDim];
   const int t = blockIdx.x;
   const int r = blockIdx.z;
   const int wave = threadIdx.x / kWave;
@@ -421,7 +422,7 @@ attention_blocks_kernel(const T* __restrict__ q, int q_stride, const T* __restri
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave][d] = to_f32(qv[d]);
   __syncthreads();
   const Query<T> a = make_query<T>(q_lds[wave], k_pages, v_pages, token_seq, positions, block_table, bt_stride, t, h,
-                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim);
+                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim, v_pitch);
   const int j0 = a.lo - a.lo % kWave + r * kWave;
   if (j0 > a.p || !active) return;  // (uniform per wave)
   float m_b, l_b, o_b[kChanPerLane];
@@ -494,26 +495,29 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
                                    const int32_t* positions, const int32_t* block_table, int bt_stride,
                                    int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
                                    int page_size, int window, float scale, float softcap, int chunk,
-                                   const float* sinks, int v_dim, int dtype, hipStream_t stream) {
+                                   const float* sinks, int v_dim, int v_pitch, int dtype, hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q_heads > 0 && n_kv_heads > 0 && page_size > 0 && bt_stride > 0,
              "attention: bad sizes");
   TL_REQUIRE(n_q_heads % n_kv_heads == 0, "attention: %d query heads are not a multiple of %d kv heads",
              n_q_heads, n_kv_heads);
-  if (head_dim <= 0 || head_dim > kMaxHeadDim)
-    return tl_fail(TL_ERR_UNSUPPORTED, "attention: head_dim=%d outside 1..%d", head_dim, kMaxHeadDim);
+  if (head_dim <= 0 || head_dim > kMaxKeyDim)
+    return tl_fail(TL_ERR_UNSUPPORTED, "attention: head_dim=%d outside 1..%d", head_dim, kMaxKeyDim);
+  if (v_pitch <= 0) v_pitch = v_dim;  // value rows lie side by side
+  TL_REQUIRE(v_pitch >= v_dim, "attention: value rows %d elements apart hold no %d channels", v_pitch, v_dim);
   TL_REQUIRE(window >= 0 && chunk >= 0, "attention: window=%d and chunk=%d must be >= 0", window, chunk);
   if (v_dim <= 0 || v_dim > kMaxHeadDim)
     return tl_fail(TL_ERR_UNSUPPORTED, "attention: values of head size %d outside 1..%d", v_dim, kMaxHeadDim);
   if (n_tokens == 0) return TL_OK;
   dim3 grid(n_tokens, (n_q_heads + kWavesPerBlock - 1) / kWavesPerBlock);
   // rows of the pages start at multiples of head_dim elements from an allocation's start
-  const bool vec = head_dim % 4 == 0 && v_dim % 4 == 0 && ((uintptr_t)k_pages % 16) == 0 && ((uintptr_t)v_pages % 16) == 0;
+  const bool vec = head_dim % 4 == 0 && v_dim % 4 == 0 && v_pitch % 4 == 0 && ((uintptr_t)k_pages % 16) == 0 && ((uintptr_t)v_pages % 16) == 0;
   // prompt portions: tokens and heads that read the same keys share them through LDS (same bits)
-  if (n_tokens >= kTileMinTokens) {
+  const size_t tile_lds = ((size_t)kTileWaves * head_dim + (size_t)kWave * (head_dim + v_dim + 2 * kTilePad)) * sizeof(float);
+  if (n_tokens >= kTileMinTokens && tile_lds <= (size_t)tl_device_facts().lds_bytes) {  // (heads too large for the tiles walk alone: the same bits)
     const int group = n_q_heads / n_kv_heads;
     const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
     const int qt = kTileWaves / hb;
-    const size_t lds = ((size_t)kTileWaves * head_dim + (size_t)kWave * (head_dim + v_dim + 2 * kTilePad)) * sizeof(float);
+    const size_t lds = tile_lds;
     dim3 tgrid((n_tokens + qt - 1) / qt, (n_q_heads + hb - 1) / hb);
 #define TL_TILE_LAUNCH_CH(T, VEC, CH)                                                                            \
   do {                                                                                                           \
@@ -525,7 +529,7 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
     attention_tile_kernel<T, VEC, CH><<<tgrid, kTileWaves * kWave, lds, stream>>>(                               \
         (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions,  \
         block_table, bt_stride, n_tokens, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, hb, softcap, \
-        chunk, sinks, v_dim);                                                                                    \
+        chunk, sinks, v_dim, v_pitch);                                                                           \
   } while (0)
 #define TL_TILE_LAUNCH(T, VEC)                                                                                   \
   do {                                                                                                           \
@@ -550,7 +554,7 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
 #define TL_ATTN_LAUNCH(T, VEC)                                                                              \
   attention_generic_kernel<T, VEC><<<grid, kWavesPerBlock * kWave, 0, stream>>>(                            \
       (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions, \
-      block_table, bt_stride, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, sinks, v_dim)
+      block_table, bt_stride, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, sinks, v_dim, v_pitch)
   if (dtype == TL_F32) {
     if (vec) TL_ATTN_LAUNCH(float, true);
     else TL_ATTN_LAUNCH(float, false);
@@ -573,14 +577,16 @@ TL_EXPORT int tl_attention_generic_split(const void* q, int q_stride, void* out,
                                          const int32_t* positions, const int32_t* block_table, int bt_stride,
                                          int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
                                          int page_size, int window, float scale, float softcap, int chunk,
-                                         const float* sinks, int v_dim, int dtype, int max_blocks,
+                                         const float* sinks, int v_dim, int v_pitch, int dtype, int max_blocks,
                                          float* partials, hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q_heads > 0 && n_kv_heads > 0 && page_size > 0 && bt_stride > 0,
              "attention: bad sizes");
   TL_REQUIRE(n_q_heads % n_kv_heads == 0, "attention: %d query heads are not a multiple of %d kv heads",
              n_q_heads, n_kv_heads);
-  if (head_dim <= 0 || head_dim > kMaxHeadDim)
-    return tl_fail(TL_ERR_UNSUPPORTED, "attention: head_dim=%d outside 1..%d", head_dim, kMaxHeadDim);
+  if (head_dim <= 0 || head_dim > kMaxKeyDim)
+    return tl_fail(TL_ERR_UNSUPPORTED, "attention: head_dim=%d outside 1..%d", head_dim, kMaxKeyDim);
+  if (v_pitch <= 0) v_pitch = v_dim;  // value rows lie side by side
+  TL_REQUIRE(v_pitch >= v_dim, "attention: value rows %d elements apart hold no %d channels", v_pitch, v_dim);
   TL_REQUIRE(window >= 0 && chunk >= 0, "attention: window=%d and chunk=%d must be >= 0", window, chunk);
   if (v_dim <= 0 || v_dim > kMaxHeadDim)
     return tl_fail(TL_ERR_UNSUPPORTED, "attention: values of head size %d outside 1..%d", v_dim, kMaxHeadDim);
@@ -590,12 +596,12 @@ TL_EXPORT int tl_attention_generic_split(const void* q, int q_stride, void* out,
   const int head_blocks = (n_q_heads + kWavesPerBlock - 1) / kWavesPerBlock;
   dim3 grid(n_tokens, head_blocks, max_blocks);
   dim3 grid_join(n_tokens, head_blocks);
-  const bool vec = head_dim % 4 == 0 && v_dim % 4 == 0 && ((uintptr_t)k_pages % 16) == 0 && ((uintptr_t)v_pages % 16) == 0;
+  const bool vec = head_dim % 4 == 0 && v_dim % 4 == 0 && v_pitch % 4 == 0 && ((uintptr_t)k_pages % 16) == 0 && ((uintptr_t)v_pages % 16) == 0;
 #define TL_ATTN_LAUNCH(T, VEC)                                                                                  \
   do {                                                                                                          \
     attention_blocks_kernel<T, VEC><<<grid, kWavesPerBlock * kWave, 0, stream>>>(                               \
         (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions, block_table, bt_stride, \
-        n_q_heads, n_kv_heads, head_dim, page_size, window, scale, partials, max_blocks, softcap, chunk, v_dim); \
+        n_q_heads, n_kv_heads, head_dim, page_size, window, scale, partials, max_blocks, softcap, chunk, v_dim, v_pitch); \
     int rc = tl_check_launch("attention_blocks");                                                               \
     if (rc != TL_OK) return rc;                                                                                 \
     attention_join_kernel<T><<<grid_join, kWavesPerBlock * kWave, 0, stream>>>(                                 \

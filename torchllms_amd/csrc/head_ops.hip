@@ -1,0 +1,347 @@
+// Kernels of layers whose branches are normed on their way into a 32-bit residual stream, and of attention
+// layers that prepare their heads before the scores: a weighted RMS norm per query and key head, rotation of
+// a part of the head, a query factor that grows with the logarithm of the position, values mixed with those
+// of an earlier layer, gates on the heads' outputs, queries and outputs of attention through a latent, and a
+// cap on the logits.  Statistics, factors, gates and the stream are 32-bit; every result is rounded once.
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+
+// ----------------------------------------------------------------------------- heads before the scores
+// rows: [n_tokens, row_stride], a row = Hq query heads of dk | Hkv key heads of dk | Hkv value heads of dv |
+// whatever follows (left alone).  One wave a head:
+//   query and key heads: the first norm_dims channels become x / sqrt(mean(x^2) + eps) * w (w given; q_w for
+//     queries, k_w for keys), the channels rot_off .. rot_off + rot - 1 are rotated by the step's table of
+//     cosines and sines (pairing 0: (2i, 2i+1); 1: (i, i + rot/2)), queries are multiplied by
+//     1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) at position p (temp_coef 0: not);
+//   value heads: v <- (1 - lam) v + lam v_first (v_first given), written back in place.
+// Queries go back in place; keys and values go to their pages [page][Hkv][P][dk] and [..][dv] at
+// slot_mapping[t] (keys in place too when there are no pages).
+constexpr int kPrepWaves = 4;
+constexpr int kPrepChan = 8;  // channels a lane holds: heads of up to 512
+
+template <typename T>
+struct PrepArgs {
+  T* rows;
+  int row_stride, n_q, n_kv, dk, dv;
+  const float* q_w;
+  const float* k_w;
+  int norm_dims;
+  float eps;
+  const float2* cos_sin;
+  int rot_off, rot, pairing;
+  const int32_t* positions;
+  float temp_coef;
+  int temp_every;
+  const T* v_first;
+  int v_first_stride;
+  const float* lam;
+  T* k_pages;
+  T* v_pages;
+  const int32_t* slot_mapping;
+  int page_size;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const PrepArgs<T> a) {
+  __shared__ float turned[kPrepWaves][kPrepChan * kWave];
+  const int t = blockIdx.x;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int unit = blockIdx.y * kPrepWaves + wave;
+  const int n_units = a.n_q + a.n_kv + (a.dv > 0 ? a.n_kv : 0);
+  const bool live = unit < n_units;
+  const bool is_q = live && unit < a.n_q;
+  const bool is_k = live && !is_q && unit < a.n_q + a.n_kv;
+  const bool is_v = live && !is_q && !is_k;
+  T* base = a.rows + (size_t)t * a.row_stride;
+  const int slot = a.slot_mapping ? a.slot_mapping[t] : -1;
+  const bool store = a.k_pages != nullptr && slot >= 0;
+  const size_t page = store ? slot / a.page_size : 0;
+  const int off = store ? slot % a.page_size : 0;
+  const int width = is_v ? a.dv : a.dk;
+  T* head = is_v ? base + (size_t)(a.n_q + a.n_kv) * a.dk + (size_t)(unit - a.n_q - a.n_kv) * a.dv
+                 : base + (size_t)(live ? unit : 0) * a.dk;
+  float val[kPrepChan];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < kPrepChan; ++c) {
+    const int d = lane + c * kWave;
+    val[c] = (live && d < width) ? to_f32(head[d]) : 0.f;
+    if (d < a.norm_dims) ss += val[c] * val[c];
+  }
+  const float* w = is_q ? a.q_w : (is_k ? a.k_w : nullptr);
+  if (w != nullptr) {  // (uniform per wave)
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)a.norm_dims + a.eps);
+#pragma unroll
+    for (int c = 0; c < kPrepChan; ++c) {
+      const int d = lane + c * kWave;
+      if (d < a.norm_dims) val[c] = val[c] * inv * w[d];
+    }
+  }
+  // rotation: every lane needs its partner's channel as it is after the norm
+  const bool turns = (is_q || is_k) && a.rot > 0;
+#pragma unroll
+  for (int c = 0; c < kPrepChan; ++c) turned[wave][lane + c * kWave] = val[c];
+  __syncthreads();
+  if (turns) {
+    const int rh = a.rot / 2;
+#pragma unroll
+    for (int c = 0; c < kPrepChan; ++c) {
+      const int d = lane + c * kWave;
+      const int r = d - a.rot_off;
+      if (d < width && r >= 0 && r < a.rot) {
+        int i, partner;
+        bool first;
+        if (a.pairing == 0) {
+          i = r / 2; first = (r % 2) == 0; partner = first ? d + 1 : d - 1;
+        } else {
+          first = r < rh; i = first ? r : r - rh; partner = first ? d + rh : d - rh;
+        }
+        const float o = turned[wave][partner];
+        const float2 cs = a.cos_sin[(size_t)t * rh + i];
+        val[c] = first ? val[c] * cs.x - o * cs.y : val[c] * cs.x + o * cs.y;
+      }
+    }
+  }
+  if (!live) return;
+  if (is_q) {
+    float f = 1.0f;
+    if (a.temp_coef != 0.f) f = 1.0f + a.temp_coef * logf((float)((a.positions[t] + 1) / a.temp_every + 1));
+#pragma unroll
+    for (int c = 0; c < kPrepChan; ++c) {
+      const int d = lane + c * kWave;
+      if (d < width) head[d] = from_f32<T>(val[c] * f);
+    }
+    return;
+  }
+  if (is_k) {
+    if (a.k_pages != nullptr && !store) return;  // a token without a slot keeps nothing
+    T* dst = store ? a.k_pages + ((page * a.n_kv + (unit - a.n_q)) * a.page_size + off) * a.dk : head;
+#pragma unroll
+    for (int c = 0; c < kPrepChan; ++c) {
+      const int d = lane + c * kWave;
+      if (d < width) dst[d] = from_f32<T>(val[c]);
+    }
+    return;
+  }
+  // a value head
+  const int g = unit - a.n_q - a.n_kv;
+  if (a.v_first != nullptr) {
+    const float lam = a.lam[0];
+    const T* vf = a.v_first + (size_t)t * a.v_first_stride + (size_t)g * a.dv;
+#pragma unroll
+    for (int c = 0; c < kPrepChan; ++c) {
+      const int d = lane + c * kWave;
+      if (d < width) {
+        val[c] = (1.0f - lam) * val[c] + lam * to_f32(vf[d]);
+        head[d] = from_f32<T>(val[c]);
+      }
+    }
+  }
+  if (store && a.v_pages != nullptr) {
+    T* dst = a.v_pages + ((page * a.n_kv + g) * a.page_size + off) * a.dv;
+#pragma unroll
+    for (int c = 0; c < kPrepChan; ++c) {
+      const int d = lane + c * kWave;
+      if (d < width) dst[d] = from_f32<T>(val[c]);
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- a normed branch into the stream
+// stream[r, :] += y[r, :] / sqrt(mean(y[r, :]^2) + eps) * w   (32-bit), and rows[r, :] = T(stream[r, :]) for the
+// next reader (rows may be null).  A block a row; the statistics in a fixed order.
+constexpr int kRowThreads = 256;
+
+template <typename T>
+__global__ void __launch_bounds__(kRowThreads)
+branch_norm_add_kernel(float* __restrict__ stream, const T* __restrict__ y, const float* __restrict__ w,
+                       T* __restrict__ rows, int hidden, float eps) {
+  __shared__ float scratch[kRowThreads / kWave];
+  const size_t r = blockIdx.x;
+  const T* yr = y + r * hidden;
+  float* sr = stream + r * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += kRowThreads) {
+    const float v = to_f32(yr[i]);
+    ss += v * v;
+  }
+  ss = block_sum<kRowThreads / kWave>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += kRowThreads) {
+    const float h = sr[i] + to_f32(yr[i]) * inv * w[i];
+    sr[i] = h;
+    if (rows) rows[r * hidden + i] = from_f32<T>(h);
+  }
+}
+
+// y[r, :] = T(x[s, :] / sqrt(mean(x[s, :]^2) + eps) * w) over `width` columns, s = rows ? rows[r] : r; x and y
+// are addressed with row strides of their own, so either may be some columns of a wider matrix.
+template <typename XT, typename T>
+__global__ void __launch_bounds__(kRowThreads)
+rmsnorm_columns_kernel(const XT* __restrict__ x, int x_stride, const int32_t* __restrict__ rows,
+                       const float* __restrict__ w, T* __restrict__ y, int y_stride, int width, float eps) {
+  __shared__ float scratch[kRowThreads / kWave];
+  const size_t r = blockIdx.x;
+  const size_t s = rows ? (size_t)rows[r] : r;
+  const XT* xr = x + s * x_stride;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += kRowThreads) {
+    const float v = to_f32(xr[i]);
+    ss += v * v;
+  }
+  ss = block_sum<kRowThreads / kWave>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += kRowThreads) y[r * y_stride + i] = from_f32<T>(to_f32(xr[i]) * inv * w[i]);
+}
+
+// ----------------------------------------------------------------------------- gates, packing, cap
+// x[t, c] *= sigmoid(g[t, c / per]) for c < width: per = 1 gates channel by channel, per = the head size gates
+// head by head.
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ x, int x_stride, const T* __restrict__ g, int g_stride, int n,
+                                    int width, int per) {
+  const size_t total = (size_t)n * width;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / width;
+    const int c = (int)(idx % width);
+    T* p = x + t * x_stride + c;
+    *p = from_f32<T>(to_f32(*p) * sigmoid_f(to_f32(g[t * g_stride + c / per])));
+  }
+}
+
+// out[t, h, :] = a[h, t, 0 .. na) | b[t, h * b_head + b_off .. + nb): the two parts of a query against a latent.
+template <typename T>
+__global__ void pack_heads_kernel(const T* __restrict__ a, int na, const T* __restrict__ b, int b_stride, int b_head,
+                                  int b_off, int nb, T* __restrict__ out, int n, int heads) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const T* ar = a + ((size_t)h * n + t) * na;
+  const T* br = b + (size_t)t * b_stride + (size_t)h * b_head + b_off;
+  T* o = out + ((size_t)t * heads + h) * (na + nb);
+  for (int i = threadIdx.x; i < na; i += blockDim.x) o[i] = ar[i];
+  for (int i = threadIdx.x; i < nb; i += blockDim.x) o[na + i] = br[i];
+}
+
+// out[t, h * d + j] = a[h, t, j] * sigmoid(g[t * g_stride + h])   (g null: no gate)
+template <typename T>
+__global__ void unpack_heads_gate_kernel(const T* __restrict__ a, T* __restrict__ out, const T* __restrict__ g,
+                                         int g_stride, int n, int heads, int d) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float f = g ? sigmoid_f(to_f32(g[(size_t)t * g_stride + h])) : 1.0f;
+  const T* ar = a + ((size_t)h * n + t) * d;
+  T* o = out + ((size_t)t * heads + h) * d;
+  for (int i = threadIdx.x; i < d; i += blockDim.x) o[i] = from_f32<T>(to_f32(ar[i]) * f);
+}
+
+__global__ void softcap_kernel(float* __restrict__ z, size_t total, float cap) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x)
+    z[idx] = cap * tanhf(z[idx] / cap);
+}
+
+int elementwise_blocks(size_t total) {
+  const size_t want = (total + 255) / 256;
+  return (int)(want < 1 ? 1 : (want > 65535 ? 65535 : want));
+}
+
+}  // namespace
+
+TL_EXPORT int tl_head_prepare(void* rows, int row_stride, int n_tokens, int n_q, int n_kv, int dk, int dv,
+                              const float* q_w, const float* k_w, int norm_dims, float eps, const float* cos_sin,
+                              int rot_off, int rot, int pairing, const int32_t* positions, float temp_coef,
+                              int temp_every, const void* v_first, int v_first_stride, const float* lam,
+                              void* k_pages, void* v_pages, const int32_t* slot_mapping, int page_size, int dtype,
+                              hipStream_t stream) {
+  TL_REQUIRE(n_tokens >= 0 && n_q >= 0 && n_kv >= 0 && n_q + n_kv > 0 && dk > 0 && dv >= 0, "head_prepare: bad sizes");
+  TL_REQUIRE(dk <= kPrepChan * kWave && dv <= kPrepChan * kWave, "head_prepare: heads of %d and %d channels, at most %d", dk, dv,
+             kPrepChan * kWave);
+  TL_REQUIRE(row_stride >= (n_q + n_kv) * dk + n_kv * dv, "head_prepare: rows of %d elements do not hold the heads", row_stride);
+  TL_REQUIRE(norm_dims >= 0 && norm_dims <= dk, "head_prepare: a norm over %d of %d channels", norm_dims, dk);
+  TL_REQUIRE((q_w == nullptr && k_w == nullptr) || norm_dims > 0, "head_prepare: norm weights without channels to norm");
+  TL_REQUIRE(rot >= 0 && rot % 2 == 0 && rot_off >= 0 && rot_off + rot <= dk, "head_prepare: %d rotated channels from %d of %d", rot, rot_off, dk);
+  TL_REQUIRE(pairing == 0 || pairing == 1, "head_prepare: pairing must be 0 (interleaved) or 1 (half split)");
+  TL_REQUIRE(rot == 0 || cos_sin != nullptr, "head_prepare: rotation without a table of cosines and sines");
+  TL_REQUIRE(temp_coef == 0.f || (positions != nullptr && temp_every > 0), "head_prepare: a query factor needs positions and a positive step");
+  TL_REQUIRE(v_first == nullptr || (lam != nullptr && dv > 0 && v_first_stride >= n_kv * dv), "head_prepare: mixed values need their factor and rows of the values' width");
+  TL_REQUIRE(k_pages == nullptr || (slot_mapping != nullptr && page_size > 0 && (dv == 0 || v_pages != nullptr)), "head_prepare: pages without slots");
+  if (n_tokens == 0) return TL_OK;
+  const int units = n_q + n_kv + (dv > 0 ? n_kv : 0);
+  const dim3 grid(n_tokens, (units + kPrepWaves - 1) / kPrepWaves);
+#define TL_PREP(T)                                                                                                   \
+  do {                                                                                                               \
+    PrepArgs<T> a{(T*)rows, row_stride, n_q, n_kv, dk, dv, q_w, k_w, (q_w || k_w) ? norm_dims : 0, eps,              \
+                  (const float2*)cos_sin, rot_off, rot, pairing, positions, temp_coef, temp_every, (const T*)v_first, \
+                  v_first_stride, lam, (T*)k_pages, (T*)v_pages, slot_mapping, page_size};                           \
+    head_prepare_kernel<T><<<grid, kPrepWaves * kWave, 0, stream>>>(a);                                              \
+  } while (0)
+  if (dtype == TL_F32) TL_PREP(float);
+  else if (dtype == TL_BF16) TL_PREP(bf16_t);
+  else return tl_fail(TL_ERR_ARG, "head_prepare: unknown dtype %d", dtype);
+#undef TL_PREP
+  return tl_check_launch("head_prepare");
+}
+
+TL_EXPORT int tl_branch_norm_add(float* stream_rows, const void* y, const float* w, void* rows, int n, int hidden, float eps,
+                                 int dtype, hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && hidden > 0, "branch_norm_add: bad sizes");
+  if (n == 0) return TL_OK;
+  if (dtype == TL_F32) branch_norm_add_kernel<float><<<n, kRowThreads, 0, stream>>>(stream_rows, (const float*)y, w, (float*)rows, hidden, eps);
+  else if (dtype == TL_BF16) branch_norm_add_kernel<bf16_t><<<n, kRowThreads, 0, stream>>>(stream_rows, (const bf16_t*)y, w, (bf16_t*)rows, hidden, eps);
+  else return tl_fail(TL_ERR_ARG, "branch_norm_add: unknown dtype %d", dtype);
+  return tl_check_launch("branch_norm_add");
+}
+
+TL_EXPORT int tl_rmsnorm_columns(const void* x, int x_stride, int x_dtype, const int32_t* rows, const float* w, void* y,
+                                 int y_stride, int y_dtype, int n, int width, float eps, hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && width > 0 && x_stride >= width && y_stride >= width, "rmsnorm_columns: bad sizes");
+  if (n == 0) return TL_OK;
+#define TL_NORM(XT, T) rmsnorm_columns_kernel<XT, T><<<n, kRowThreads, 0, stream>>>((const XT*)x, x_stride, rows, w, (T*)y, y_stride, width, eps)
+  if (x_dtype == TL_F32 && y_dtype == TL_F32) TL_NORM(float, float);
+  else if (x_dtype == TL_F32 && y_dtype == TL_BF16) TL_NORM(float, bf16_t);
+  else if (x_dtype == TL_BF16 && y_dtype == TL_BF16) TL_NORM(bf16_t, bf16_t);
+  else return tl_fail(TL_ERR_ARG, "rmsnorm_columns: input dtype %d with output dtype %d", x_dtype, y_dtype);
+#undef TL_NORM
+  return tl_check_launch("rmsnorm_columns");
+}
+
+TL_EXPORT int tl_sigmoid_gate(void* x, int x_stride, const void* g, int g_stride, int n, int width, int per, int dtype,
+                              hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && width > 0 && per > 0 && x_stride >= width, "sigmoid_gate: bad sizes");
+  if (n == 0) return TL_OK;
+  const int blocks = elementwise_blocks((size_t)n * width);
+  if (dtype == TL_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, x_stride, (const float*)g, g_stride, n, width, per);
+  else if (dtype == TL_BF16) sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, x_stride, (const bf16_t*)g, g_stride, n, width, per);
+  else return tl_fail(TL_ERR_ARG, "sigmoid_gate: unknown dtype %d", dtype);
+  return tl_check_launch("sigmoid_gate");
+}
+
+TL_EXPORT int tl_pack_heads(const void* a, int na, const void* b, int b_stride, int b_head, int b_off, int nb, void* out, int n,
+                            int heads, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && heads > 0 && heads <= 65535 && na >= 0 && nb >= 0 && na + nb > 0, "pack_heads: bad sizes");
+  if (n == 0) return TL_OK;
+  const dim3 grid(n, heads);
+  if (dtype == TL_F32) pack_heads_kernel<float><<<grid, 128, 0, stream>>>((const float*)a, na, (const float*)b, b_stride, b_head, b_off, nb, (float*)out, n, heads);
+  else if (dtype == TL_BF16) pack_heads_kernel<bf16_t><<<grid, 128, 0, stream>>>((const bf16_t*)a, na, (const bf16_t*)b, b_stride, b_head, b_off, nb, (bf16_t*)out, n, heads);
+  else return tl_fail(TL_ERR_ARG, "pack_heads: unknown dtype %d", dtype);
+  return tl_check_launch("pack_heads");
+}
+
+TL_EXPORT int tl_unpack_heads_gate(const void* a, void* out, const void* g, int g_stride, int n, int heads, int d, int dtype,
+                                   hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && heads > 0 && heads <= 65535 && d > 0, "unpack_heads_gate: bad sizes");
+  if (n == 0) return TL_OK;
+  const dim3 grid(n, heads);
+  if (dtype == TL_F32) unpack_heads_gate_kernel<float><<<grid, 128, 0, stream>>>((const float*)a, (float*)out, (const float*)g, g_stride, n, heads, d);
+  else if (dtype == TL_BF16) unpack_heads_gate_kernel<bf16_t><<<grid, 128, 0, stream>>>((const bf16_t*)a, (bf16_t*)out, (const bf16_t*)g, g_stride, n, heads, d);
+  else return tl_fail(TL_ERR_ARG, "unpack_heads_gate: unknown dtype %d", dtype);
+  return tl_check_launch("unpack_heads_gate");
+}
+
+TL_EXPORT int tl_softcap(float* z, long long total, float cap, hipStream_t stream) {
+  TL_REQUIRE(total >= 0 && cap > 0.f, "softcap: bad sizes or a cap that is not positive");
+  if (total == 0) return TL_OK;
+  softcap_kernel<<<elementwise_blocks((size_t)total), 256, 0, stream>>>(z, (size_t)total, cap);
+  return tl_check_launch("softcap");
+}

@@ -36,6 +36,7 @@ CORE_SOURCES = [
     "gemm_wide.hip",
     "sampling.hip",
     "sequence_ops.hip",
+    "head_ops.hip",
 ]
 HEADERS = ["common.h", "qkv_epilogue.h", "no_alloc.h"]
 

@@ -32,8 +32,8 @@ _CORE_SIGNATURES = {
     "tl_rope_kv_write": [_P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _P],
     "tl_silu_mul": [_P, _P, _I, _I, _I, _P],
     "tl_add_bias": [_P, _P, _I, _I, _I, _I, _P],
-    "tl_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _I, _I, _P],
-    "tl_attention_generic_split": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _I, _I, _I, _P, _P],
+    "tl_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _I, _I, _I, _P],
+    "tl_attention_generic_split": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _I, _I, _I, _I, _P, _P],
     "tl_embed_scaled": [_P, _P, _P, _I, _I, _F, _I, _P],
     "tl_layernorm": [_P, _P, _P, _F, _P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _P],
     "tl_gelu_mul": [_P, _P, _I, _I, _I, _P],
@@ -41,6 +41,13 @@ _CORE_SIGNATURES = {
     "tl_causal_conv": [_P, _I, _P, _P, _P, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "tl_selective_scan": [_P, _P, _I, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P],
     "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
+    "tl_head_prepare": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _I, _I, _I, _P, _F, _I, _P, _I, _P, _P, _P, _P, _I, _I, _P],
+    "tl_branch_norm_add": [_P, _P, _P, _P, _I, _I, _F, _I, _P],
+    "tl_rmsnorm_columns": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _F, _P],
+    "tl_sigmoid_gate": [_P, _I, _P, _I, _I, _I, _I, _I, _P],
+    "tl_pack_heads": [_P, _I, _P, _I, _I, _I, _I, _P, _I, _I, _I, _P],
+    "tl_unpack_heads_gate": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "tl_softcap": [_P, _I64, _F, _P],
     "tl_gemm_f32": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _I, _P],

@@ -11,6 +11,8 @@ a module's own helpers and tables stay in the module.
 ``attention_ops``    plain, decode and prefill attention with their launch plans
 ``sequence_ops``     layer norm with a scaled sum, gated activations, unit-norm rotation with the cache
                      write, short convolutions, selective scan, gated delta rule
+``head_ops``         branches normed into a 32-bit stream, heads prepared before the scores (weighted norm, partial
+                     rotation, query factor, mixed values), gates, packing for attention through a latent, logit cap
 ``sampling_ops``     the sampling kernel
 """
 
@@ -71,6 +73,7 @@ from .products import (  # noqa: F401
 )
 from .attention_ops import (  # noqa: F401
     ATTENTION_MAX_HEAD_DIM,
+    ATTENTION_MAX_KEY_DIM,
     DECODE_HEAD_DIMS,
     PREFILL_HEAD_DIMS,
     PREFILL_SPLIT_ALWAYS,
@@ -100,6 +103,16 @@ from .sequence_ops import (  # noqa: F401
     rope_norm_kv_write,
     selective_scan,
     state_region,
+)
+from .head_ops import (  # noqa: F401
+    HEAD_PREPARE_MAX_DIM,
+    branch_norm_add,
+    head_prepare,
+    pack_heads,
+    rmsnorm_columns,
+    sigmoid_gate_,
+    softcap_,
+    unpack_heads_gate,
 )
 from .sampling_ops import (  # noqa: F401
     philox_uniform,

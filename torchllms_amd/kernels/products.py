@@ -27,8 +27,9 @@ from .base import (  # noqa: F401
 )
 from .elementwise_ops import add_bias_, rmsnorm, rope_kv_write, rope_table, silu_mul  # noqa: F401
 
-def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """``x @ w.T`` in true 32-bit arithmetic; x [m, k], w [n, k], both float32."""
+def gemm_f32(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``x @ w.T`` in true 32-bit arithmetic; x [m, k], w [n, k], both float32 and row-major (rows may lie apart);
+    ``out``: a row-major float32 [m, n] to write into (some columns of a wider matrix will do)."""
     _gpu(x, w)
     if x.dtype != torch.float32 or w.dtype != torch.float32:
         raise KernelError("gemm_f32 takes float32 tensors")
@@ -36,7 +37,10 @@ def gemm_f32(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         raise KernelError(f"gemm_f32: shapes {tuple(x.shape)} x {tuple(w.shape)}^T do not match")
     m, k = x.shape
     n = w.shape[0]
-    out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=x.device)
+    elif out.shape != (m, n) or out.dtype != torch.float32 or out.stride(1) != 1 or not out.is_cuda:
+        raise KernelError(f"gemm_f32: out must be a row-major float32 [{m}, {n}] GPU tensor")
     check(core().tl_gemm_f32(x.data_ptr(), x.stride(0), w.data_ptr(), w.stride(0), out.data_ptr(), out.stride(0), m, n, k, _stream()))
     return out
 

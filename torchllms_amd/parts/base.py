@@ -34,7 +34,8 @@ class ParamSpec:
     ``kind``: "matrix" (kept in the model's compute dtype), "vector" (compute dtype, but a
     tensor stored in 32-bit stays in 32-bit), "int" (an integer table, kept as int32).
     ``init``: how the random-weights mode fills it: "normal" N(0, 0.02), "ones", "zeros", "conv" and "wide" (N(0, 0.5):
-    the taps of a short convolution, a projection from very few inputs).
+    the taps of a short convolution, a projection from very few inputs), "fraction" (uniform between 0.25 and 0.75: a
+    mixing factor).
     """
 
     shape: Tuple[int, ...]
@@ -51,6 +52,9 @@ class KVNeed:
     ``page_size`` (tokens per page) and ``dtype`` ("float32", "bfloat16") are the engine's own
     unless the mixer asks for others; layers that ask for the same form one group of pages.
     ``v_head_dim``: the head size of the values when it is not that of the keys.
+    ``values_in_keys``: a token's value is the first ``v_head_dim`` channels of its key row (attention through a
+    latent: the latent is the value and, with the rotated part behind it, the key), so no value pages are kept and
+    a mixer's ``v_pages`` is its ``k_pages``.
     """
 
     num_kv_heads: int
@@ -59,6 +63,7 @@ class KVNeed:
     page_size: Optional[int] = None
     dtype: Optional[str] = None
     v_head_dim: Optional[int] = None
+    values_in_keys: bool = False
 
 
 @dataclass(frozen=True)

@@ -59,3 +59,61 @@ class ParallelMixerBlock(_Parallel):
 
     def branches(self, y, ctx, cache):
         return [self.mix.forward(y, ctx, cache["mix"])]
+
+
+class _BranchNorm(Block):
+    """Layers whose norms stand behind the branches: every branch reads the residual stream itself and its
+    output is normed on the way into the stream, ``x <- x + norm(branch(x))``, one branch after the other.
+    The stream is 32-bit whatever the model's dtype (an embedding with ``stream_dtype="float32"`` opens it, norms
+    with ``stream_dtype="float32"`` keep it); the rows a branch reads are the stream rounded to the model's
+    dtype, which the norm's kernel leaves beside the sum.  Nothing is handed on unapplied."""
+
+    graph_safe = True
+    _ROWS = "stream_rows"  # in ctx.scratch: (the stream the rows were made from, the rows in the model's dtype)
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.dtype = None
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        matrices = [v for v in tensors.values() if v.dim() == 2]
+        self.dtype = matrices[0].dtype if matrices else next(iter(tensors.values())).dtype
+
+    def rows_of(self, h, ctx):
+        kept = ctx.scratch.get(self._ROWS)
+        if kept is not None and kept[0] is h:
+            return kept[1]
+        return h if h.dtype == self.dtype else h.to(self.dtype)
+
+    def keep_rows(self, h, rows, ctx):
+        ctx.scratch[self._ROWS] = (h, rows)
+
+
+@BLOCKS.register("branch_norm")
+class BranchNormBlock(_BranchNorm):
+    """``x <- x + norm1(mix(x)); x <- x + norm2(mlp(x))``."""
+
+    SLOTS = {"norm1": "norm", "norm2": "norm", "mix": "mixer", "mlp": "feed_forward"}
+
+    def forward(self, h, delta, ctx, cache):
+        if delta is not None:
+            h = h + ops.resolved(delta).float()
+        h, x = self.norm1.forward_branch(h, self.mix.forward(self.rows_of(h, ctx), ctx, cache["mix"]))
+        h, x = self.norm2.forward_branch(h, self.mlp.forward(x, ctx))
+        self.keep_rows(h, x, ctx)
+        return h, None
+
+
+@BLOCKS.register("branch_norm_mixer")
+class BranchNormMixerBlock(_BranchNorm):
+    """The same layer without a feed-forward: ``x <- x + norm1(mix(x))``."""
+
+    SLOTS = {"norm1": "norm", "mix": "mixer"}
+
+    def forward(self, h, delta, ctx, cache):
+        if delta is not None:
+            h = h + ops.resolved(delta).float()
+        h, x = self.norm1.forward_branch(h, self.mix.forward(self.rows_of(h, ctx), ctx, cache["mix"]))
+        self.keep_rows(h, x, ctx)
+        return h, None

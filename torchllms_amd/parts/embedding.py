@@ -44,14 +44,18 @@ class TokenEmbedding(Embedding):
 @HEADS.register("lm_head")
 class LMHead(Head):
     """``logits = x W^T`` with W [vocab, hidden], no bias; with ``tied`` W is the embedding
-    matrix (reference: torchllms/models/networks.py:804-809,1047).  Logits are returned in 32-bit."""
+    matrix (reference: torchllms/models/networks.py:804-809,1047).  Logits are returned in 32-bit.
+    ``softcap`` c > 0: the logits become ``c * tanh(logits / c)``."""
 
     graph_safe = True
 
-    def __init__(self, vocab_size: int, hidden_size: int, tied: bool):
+    def __init__(self, vocab_size: int, hidden_size: int, tied: bool, softcap: float = 0.0):
+        if softcap < 0:
+            raise ValueError(f"lm_head: softcap {softcap!r} must not be negative")
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.tied = tied
+        self.softcap = float(softcap)
         self.weight: Optional[torch.Tensor] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -74,4 +78,9 @@ class LMHead(Head):
         return ["weight"] if self.tied else []
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.linear(x, self.weight, out_dtype=torch.float32)
+        logits = ops.linear(x, self.weight, out_dtype=torch.float32)
+        if self.softcap > 0:
+            if not logits.is_contiguous():
+                logits = logits.contiguous()
+            ops.softcap_(logits, self.softcap)
+        return logits

@@ -1,0 +1,163 @@
+"""Attention through a latent: keys and values of all heads are expanded from one compressed vector per token."""
+
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..config.spec import PartSpec
+from ..kernels import ops
+from ..kernels.attention import paged_attention
+from .base import MIXERS, POSITIONS, KVNeed, Mixer, ParamSpec
+
+
+@MIXERS.register("latent_attention")
+class LatentAttention(Mixer):
+    """Every token leaves one latent ``c`` of ``kv_rank`` channels (a projection of the layer's input, RMS-normed
+    with a weight) and one rotated key part of ``rot_dim`` channels that all heads share.  Head h's key is
+    ``[W_uk[h] c | rotated part]``, its value ``W_uv[h] c``; queries come through a normed latent of their own
+    (``q_rank`` channels) as ``[dim unrotated | rot_dim rotated]`` per head.  Causal softmax attention, an optional
+    gate per head (the sigmoid of a projection of the layer's input), the output projection.
+
+    Only ``c`` and the rotated part are cached, as one key row ``[c | rotated part]`` of a single kv head; the
+    expansions never happen per cached token.  With ``q' = W_uk[h]^T q_unrotated`` the score of head h is
+    ``q' . c + q_rotated . k_rotated``, and the head's output is ``W_uv[h] (sum_j p_j c_j)``: attention of H query
+    heads of ``kv_rank + rot_dim`` channels over one kv head whose values are the first ``kv_rank`` channels of
+    its keys (``KVNeed.values_in_keys``), with one small product per head before and after it.
+    """
+
+    graph_safe = True
+
+    def __init__(
+        self,
+        hidden_size: int,
+        num_heads: int,
+        head_dim: int,
+        rot_dim: int,
+        v_head_dim: int,
+        q_rank: int,
+        kv_rank: int,
+        softmax_scale: float,
+        norm_eps: float,
+        position: PartSpec,
+        head_gate: bool = False,
+        kv_page_size: Optional[int] = None,
+    ):
+        if rot_dim < 0 or rot_dim % 2:
+            raise ValueError(f"latent attention: {rot_dim} rotated channels (even, not negative)")
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.head_dim = head_dim
+        self.rot_dim = rot_dim
+        self.v_head_dim = v_head_dim
+        self.q_rank = q_rank
+        self.kv_rank = kv_rank
+        self.softmax_scale = float(softmax_scale)
+        self.norm_eps = float(norm_eps)
+        self.head_gate = bool(head_gate)
+        self.kv_page_size = kv_page_size
+        self.position = POSITIONS.build(position)
+        self.w_down: Optional[torch.Tensor] = None   # [q_rank + kv_rank + rot_dim + gates, hidden]
+        self.w_uq: Optional[torch.Tensor] = None     # [H * (dim + rot_dim), q_rank]
+        self.w_uk_t: Optional[torch.Tensor] = None   # [H, kv_rank, dim]: q' = W_uk[h]^T q
+        self.w_uv: Optional[torch.Tensor] = None     # [H, vdim, kv_rank]
+        self.wo: Optional[torch.Tensor] = None
+        self.q_norm: Optional[torch.Tensor] = None
+        self.kv_norm: Optional[torch.Tensor] = None
+
+    @property
+    def key_dim(self) -> int:
+        """Channels of a cached row, and of a query against it."""
+        return self.kv_rank + self.rot_dim
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        H, d, r, dv = self.num_heads, self.head_dim, self.rot_dim, self.v_head_dim
+        specs = {
+            "dq.weight": ParamSpec((self.q_rank, self.hidden_size)),
+            "dq_norm.weight": ParamSpec((self.q_rank,), kind="vector", init="ones"),
+            "uq.weight": ParamSpec((H * (d + r), self.q_rank)),
+            "dkv.weight": ParamSpec((self.kv_rank + r, self.hidden_size)),
+            "dkv_norm.weight": ParamSpec((self.kv_rank,), kind="vector", init="ones"),
+            "uk.weight": ParamSpec((H * d, self.kv_rank)),
+            "uv.weight": ParamSpec((H * dv, self.kv_rank)),
+            "wo.weight": ParamSpec((self.hidden_size, H * dv)),
+        }
+        if self.head_gate:
+            specs["wg.weight"] = ParamSpec((H, self.hidden_size))
+        return specs
+
+    def check_sizes(self, dtype: torch.dtype) -> None:
+        if not 0 < self.kv_rank <= ops.ATTENTION_MAX_HEAD_DIM:
+            raise ValueError(f"latent attention: a latent of {self.kv_rank} channels; the attention kernel takes values of up to {ops.ATTENTION_MAX_HEAD_DIM}")
+        if self.key_dim > min(ops.ATTENTION_MAX_KEY_DIM, ops.HEAD_PREPARE_MAX_DIM):
+            raise ValueError(f"latent attention: rows of {self.key_dim} channels (latent and rotated part); the kernels take "
+                             f"{min(ops.ATTENTION_MAX_KEY_DIM, ops.HEAD_PREPARE_MAX_DIM)}")
+        if self.head_dim + self.rot_dim > ops.HEAD_PREPARE_MAX_DIM:
+            raise ValueError(f"latent attention: query heads of {self.head_dim + self.rot_dim} channels, at most {ops.HEAD_PREPARE_MAX_DIM}")
+        if self.rot_dim and getattr(self.position, "rotary_dim", 0) != self.rot_dim:
+            raise ValueError("latent attention: the position encoding must rotate exactly the rotated part")
+
+    def cache_need(self):
+        return KVNeed(num_kv_heads=1, head_dim=self.key_dim, window=0, page_size=self.kv_page_size, v_head_dim=self.kv_rank,
+                      values_in_keys=True)
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        H, d, dv = self.num_heads, self.head_dim, self.v_head_dim
+        down = [tensors["dq.weight"], tensors["dkv.weight"]] + ([tensors["wg.weight"]] if self.head_gate else [])
+        self.w_down = torch.cat(down, dim=0).contiguous()
+        self.w_uq = tensors["uq.weight"].contiguous()
+        self.w_uk_t = tensors["uk.weight"].reshape(H, d, self.kv_rank).transpose(1, 2).contiguous()
+        self.w_uv = tensors["uv.weight"].reshape(H, dv, self.kv_rank).contiguous()
+        self.wo = tensors["wo.weight"].contiguous()
+        self.q_norm = tensors["dq_norm.weight"].float().contiguous()
+        self.kv_norm = tensors["dkv_norm.weight"].float().contiguous()
+        self.position.to(self.wo.device)
+
+    def linear_weights(self):
+        return [self.w_down, self.w_uq, (self.wo, "sum")]
+
+    def _per_head(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """``out[h] = x[:, h, :] @ w[h].T`` as [H, n, rows of w[h]]: x a view [n, H, k] whose rows may lie apart."""
+        H, n = w.shape[0], x.shape[0]
+        if x.dtype == torch.float32:
+            # the 32-bit product kernel, head by head: every sum in an order that the batch does not change
+            out = torch.empty((H, n, w.shape[1]), dtype=torch.float32, device=x.device)
+            for h in range(H):
+                ops.gemm_f32(x[:, h, :], w[h], out=out[h])
+            return out
+        return torch.bmm(x.transpose(0, 1), w.transpose(1, 2))
+
+    def forward(self, x, ctx, cache):
+        H, d, r, R = self.num_heads, self.head_dim, self.rot_dim, self.kv_rank
+        g = cache.group
+        rot = self.position.rotary_args()
+        table = None
+        if r > 0:
+            key = ("rope_table", rot.inv_freq.data_ptr())
+            table = ctx.scratch.get(key)
+            if table is None:
+                table = ctx.scratch[key] = ops.rope_table(ctx.positions, rot.inv_freq)
+        pairing = rot.pairing if rot else 0
+        x = ops.resolved(x)
+        n = x.shape[0]
+        down = ops.linear(x, self.w_down)  # query latent | latent | shared rotated key part | gates
+        # the latent is normed, the shared part rotated, and the row goes to its page as one key
+        ops.head_prepare(
+            down[:, self.q_rank :], 0, 1, R + r, 0, k_norm=self.kv_norm, norm_dims=R, eps=self.norm_eps, cos_sin=table,
+            rot_offset=R, rot_dims=r, pairing=pairing, k_pages=cache.k_pages if cache.writes else None,
+            slot_mapping=ctx.slot_mappings[g] if cache.writes else None, page_size=cache.page_size if cache.writes else 0,
+        )
+        cq = ops.rmsnorm_columns(down[:, : self.q_rank], self.q_norm, self.norm_eps, x.dtype)
+        q = ops.linear(cq, self.w_uq)  # [n, H * (d + r)]
+        if r > 0:
+            ops.head_prepare(q, H, 0, d + r, 0, cos_sin=table, rot_offset=d, rot_dims=r, pairing=pairing)
+        q_lat = self._per_head(q.view(n, H, d + r)[:, :, :d], self.w_uk_t)       # [H, n, R]
+        queries = ops.pack_heads(q_lat, q, d + r, d, r)                           # [n, H * (R + r)]
+        mixed = paged_attention(
+            queries, H, 1, R + r, cache.k_pages, cache.v_pages, ctx, g, 0, self.softmax_scale, v_head_dim=R, values_in_keys=True,
+        )                                                                         # [n, H * R]: the heads' mixed latents
+        heads = self._per_head(mixed.view(n, H, R), self.w_uv)                    # [H, n, dv]
+        gates = down[:, self.q_rank + R + r :] if self.head_gate else None
+        out = ops.unpack_heads_gate(heads.contiguous(), gates)
+        return ops.linear_to_sum(out, self.wo, may_wait=True)

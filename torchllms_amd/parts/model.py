@@ -14,6 +14,7 @@ from . import attention as _attention  # noqa: F401
 from . import blocks as _blocks  # noqa: F401
 from . import embedding as _embedding  # noqa: F401
 from . import feed_forward as _feed_forward  # noqa: F401
+from . import latent as _latent  # noqa: F401
 from . import norms as _norms  # noqa: F401
 from . import positions as _positions  # noqa: F401
 from . import recurrent as _recurrent  # noqa: F401

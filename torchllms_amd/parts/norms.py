@@ -13,18 +13,29 @@ from .base import NORMS, Norm, ParamSpec
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
     """``y = cast(x32 * rsqrt(mean(x32^2) + eps)) * weight``: statistics and scaling in 32-bit,
-    the weight multiply after the cast back (reference: torchllms/models/networks.py:186-200)."""
+    the weight multiply after the cast back (reference: torchllms/models/networks.py:186-200).
+
+    ``stream_dtype`` "float32": the norm works beside a 32-bit residual stream whatever the model's dtype.
+    Then ``y = cast(x32 * rsqrt(mean(x32^2) + eps) * weight32)``, rounded once; it reads rows of the stream or of
+    the model's dtype and hands on rows of the model's dtype, and ``forward_branch`` adds a normed branch to the
+    stream (``stream += norm(branch)``), which is what a block that norms its branches' outputs calls."""
 
     graph_safe = True
     takes_split_sums = True  # ops.rmsnorm adds the slices of a split product while it reads them
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, stream_dtype: Optional[str] = None):
+        if stream_dtype not in (None, "float32"):
+            raise ValueError(f"rmsnorm: stream_dtype {stream_dtype!r} (None: the model's dtype, or \"float32\")")
         self.size = size
         self.eps = float(eps)
+        self.stream_dtype = stream_dtype
+        self.takes_split_sums = stream_dtype is None
         self.weight: Optional[torch.Tensor] = None
+        self.out_dtype: Optional[torch.dtype] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.size,), kind="vector", init="ones")}
+        # (beside a 32-bit stream the vector follows the model's dtype, which is the dtype of the normed rows)
+        return {"weight": ParamSpec((self.size,), kind="vector" if self.stream_dtype is None else "matrix", init="ones")}
 
     def check_sizes(self, dtype: torch.dtype) -> None:
         if not 0 < self.size <= ops.rmsnorm_max_hidden():
@@ -32,11 +43,27 @@ class RMSNorm(Norm):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self.weight = tensors["weight"].contiguous()
+        if self.stream_dtype is not None:
+            self.out_dtype = self.weight.dtype
+            self.weight = self.weight.float().contiguous()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.stream_dtype is not None:
+            return ops.rmsnorm_columns(x, self.weight, self.eps, self.out_dtype)
         return ops.rmsnorm(x, self.weight, self.eps)
 
+    def forward_branch(self, stream: torch.Tensor, branch, want_rows: bool = True):
+        """``stream += norm(branch)`` in place and in 32-bit; returns ``(stream, its new rows in the model's dtype)``
+        (the rows are None with ``want_rows`` False: nobody reads them)."""
+        if self.stream_dtype is None:
+            raise ValueError("rmsnorm: forward_branch needs the 32-bit residual stream (stream_dtype=\"float32\")")
+        return stream, ops.branch_norm_add(stream, ops.resolved(branch), self.weight, self.eps, want_rows=want_rows)
+
     def forward_add(self, h: torch.Tensor, delta: Optional[torch.Tensor]):
+        if self.stream_dtype is not None:
+            if delta is not None:
+                h = h + ops.resolved(delta).float()
+            return h, self.forward(h)
         if delta is None:
             return h, ops.rmsnorm(h, self.weight, self.eps)
         return ops.rmsnorm(h, self.weight, self.eps, delta=delta, return_sum=True)
@@ -49,6 +76,10 @@ class RMSNorm(Norm):
         return self.forward_add(h, delta)
 
     def forward_rows(self, h: torch.Tensor, delta: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
+        if self.stream_dtype is not None:
+            if delta is not None:
+                h = h + ops.resolved(delta).float()
+            return ops.rmsnorm_columns(h, self.weight, self.eps, self.out_dtype, rows=rows)
         return ops.rmsnorm(h, self.weight, self.eps, delta=delta, rows=rows)
 
 

@@ -155,3 +155,29 @@ def taluvik_name_rules(cfg) -> List[NameRule]:
         else:
             rules += [NameRule(p + n, p + n) for n in recurrent]
     return rules
+
+
+def vobolorn_name_rules(cfg) -> List[NameRule]:
+    """Vobolorn checkpoints name a layer's tensors ``l<i>.norm1``, ``l<i>.norm2``, ``l<i>.mix.<tensor>`` (a bias
+    is the tensor's name with ``.b``, a norm inside the mixer ``<tensor>.norm``) and ``l<i>.mlp.{gate,up,down}``.
+    The rules are written per layer, from the layer's type: the mixers share names (every one has an ``o``)."""
+    L = "l{}."
+    rules = [
+        NameRule("embed", "embed.weight"),
+        NameRule("final.norm", "final_norm.weight"),
+        NameRule("head", "head.weight"),
+        NameRule(L + "norm1", L + "norm1.weight"),
+        NameRule(L + "norm2", L + "norm2.weight"),
+        NameRule(L + "mlp.gate", L + "mlp.w1.weight"),
+        NameRule(L + "mlp.up", L + "mlp.w3.weight"),
+        NameRule(L + "mlp.down", L + "mlp.w2.weight"),
+    ]
+    grouped = {"q": "wq.weight", "k": "wk.weight", "v": "wv.weight", "o": "wo.weight", "q.b": "wq.bias", "k.b": "wk.bias",
+               "v.b": "wv.bias", "q.norm": "q_norm.weight", "k.norm": "k_norm.weight", "vmix": "vmix", "g": "wg.weight"}
+    latent = {"dq": "dq.weight", "dq.norm": "dq_norm.weight", "uq": "uq.weight", "dkv": "dkv.weight", "dkv.norm": "dkv_norm.weight",
+              "uk": "uk.weight", "uv": "uv.weight", "g": "wg.weight", "o": "wo.weight"}
+    for i, layer in enumerate(cfg.layers):
+        p = f"l{i}.mix."
+        names = latent if layer.type == "latent_attention" else grouped
+        rules += [NameRule(p + ext, p + own) for ext, own in names.items()]
+    return rules

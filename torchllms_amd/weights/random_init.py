@@ -47,6 +47,9 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, dtype: torch.dtype, nor
     elif spec.init == "wide":
         # a projection from very few inputs (a low-rank step size): N(0, 0.02) would leave it flat
         t = torch.empty(spec.shape, dtype=torch.float32, device=device).normal_(0.0, 0.5, generator=gen)
+    elif spec.init == "fraction":
+        # a mixing factor between two things: well inside (0, 1), so that both show
+        t = torch.empty(spec.shape, dtype=torch.float32, device=device).uniform_(0.25, 0.75, generator=gen)
     elif spec.init == "zeros":
         t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
         if norm_jitter > 0:
