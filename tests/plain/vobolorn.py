@@ -103,7 +103,8 @@ def attention_mixer(h: torch.Tensor, w: Dict[str, torch.Tensor], p: str, m: dict
     if qt:
         q = q * query_temperature(S, qt["coef"], qt["every"], q.dtype).reshape(S, 1, 1)
     if m.get("v_mix"):
-        v = mix_values(v, shared.get("v_first"), w[p + "vmix"])
+        first = shared.get("v_first")
+        v = mix_values(v, first, w[p + "vmix"] if first is not None else None)  # (the first such layer's factor is unused)
         shared.setdefault("v_first", v)
     o = causal_softmax_attention(q, k, v, m["scale"]).reshape(S, H * dv)
     if gate:

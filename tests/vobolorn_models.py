@@ -1,0 +1,110 @@
+"""Small Vobolorn configurations for the tests, and model folders with random weights made from them.
+
+The configurations differ from each other in every size and constant, and in what a single model may
+happen to make equal: heads and key heads, head sizes of keys and values, the latent's sizes, layers
+with and without a feed-forward, a latent layer first, values mixed by one layer, by several, by none,
+logits capped and not, head sizes that the matrix-core attention kernels take and that they do not, a
+latent wider than the attention kernel's values."""
+
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Dict
+
+import torch
+
+
+def grouped(kind, heads, kv_heads, dim, vdim, scale, q_temp=None, v_mix=False):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale}
+    if q_temp is not None:
+        m["q_temp"] = {"coef": q_temp[0], "every": q_temp[1]}
+    if v_mix:
+        m["v_mix"] = True
+    return kind, m
+
+
+def latent(heads, dim, rot_dim, vdim, q_rank, kv_rank, scale, base=10000.0):
+    return "latent_attention", {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "q_rank": q_rank, "kv_rank": kv_rank,
+                                "scale": scale, "rot": {"base": base, "dims": rot_dim}}
+
+
+def layer(mixer, ff=None):
+    kind, m = mixer
+    return {"type": kind, "mixer": m, "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+
+
+def model(vocab, width, eps, layers, softcap=None):
+    d = {"architecture": "Vobolorn", "vocab": vocab, "width": width, "norm": {"eps": eps}, "layers": layers}
+    if softcap is not None:
+        d["logit_softcap"] = softcap
+    return d
+
+
+CONFIG_A = model(131, 64, 1e-5, [
+    layer(grouped("attention_2", 4, 2, 32, 16, 0.5, q_temp=(0.5, 7), v_mix=True), ff=80),
+    layer(latent(3, 24, 8, 20, 28, 40, 0.4), ff=48),
+    layer(grouped("attention", 4, 2, 24, 16, 0.6, v_mix=True), ff=80),
+    layer(grouped("attention_2", 2, 2, 40, 16, 0.4, q_temp=(0.2, 16), v_mix=True)),
+], softcap=12.0)
+
+CONFIG_B = model(77, 96, 1e-6, [
+    layer(latent(2, 16, 32, 48, 16, 72, 0.3, base=500.0)),
+    layer(grouped("attention", 6, 6, 48, 48, 0.35), ff=112),
+    layer(grouped("attention_2", 6, 3, 20, 36, 0.7, q_temp=(0.8, 1), v_mix=True), ff=112),
+])
+
+CONFIG_C = model(200, 128, 1e-5, [
+    layer(grouped("attention", 2, 1, 128, 128, 0.25, v_mix=True), ff=96),
+    layer(grouped("attention_2", 4, 1, 128, 128, 0.2, q_temp=(0.3, 10), v_mix=True), ff=96),
+    layer(latent(4, 32, 16, 32, 24, 288, 0.3, base=50.0), ff=64),
+    layer(grouped("attention_2", 8, 2, 64, 64, 0.3, q_temp=(1.0, 3))),
+], softcap=50.0)
+
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
+PAGE_SIZE = {"A": 8, "B": 16, "C": 4}
+
+
+def single_layer(entry: dict, width: int = 64, vocab: int = 61, softcap=None) -> dict:
+    """A model of one layer, for a mechanism alone."""
+    return model(vocab, width, 1e-5, [entry], softcap=softcap)
+
+
+#: how much a tensor of a mixer is scaled up after the random-weights mode has drawn it from N(0, 0.02) (or from
+#: N(0, 0.02) around zero for biases): projections before a norm need no scale, what stands behind one or enters a
+#: sigmoid does, or a forgotten bias, gate or rotated part would hardly show
+_SCALES = {"mix.q.b": 12.0, "mix.k.b": 12.0, "mix.v.b": 12.0, "mix.g": 12.0, "mix.uq": 20.0, "mix.uk": 20.0, "mix.dkv": 3.0}
+
+
+def make_folder(path, cfg_dict: dict, seed: int = 0, dtype=torch.bfloat16) -> Path:
+    """A model folder written by the package's random-weights mode (norm weights 1 + N(0, 0.1), mixing factors
+    between 0.25 and 0.75), then made harder on faults by the scales above."""
+    from safetensors.torch import save_file
+
+    from torchllms_amd.config.vobolorn import VobolornConfig
+    from torchllms_amd.weights import write_model_folder
+
+    folder = write_model_folder(path, VobolornConfig.from_dict(cfg_dict), seed=seed, dtype=dtype, norm_jitter=0.1)
+    _, tensors = read_folder(folder)
+    for name in list(tensors):
+        leaf = name.split(".", 1)[-1] if name.startswith("l") else name
+        if leaf in _SCALES:
+            tensors[name] = (tensors[name].float() * _SCALES[leaf]).to(dtype)
+    save_file(tensors, str(folder / "model.safetensors"), metadata={"format": "pt"})
+    return folder
+
+
+def read_folder(folder) -> (dict, Dict[str, torch.Tensor]):
+    """config.json as a dict and the tensors by their checkpoint names, read with safetensors
+    directly (not through the package's loader)."""
+    import json
+
+    from safetensors import safe_open
+
+    folder = Path(folder)
+    with open(folder / "config.json") as f:
+        cfg = json.load(f)
+    tensors = {}
+    with safe_open(str(folder / "model.safetensors"), framework="pt", device="cpu") as f:
+        for name in f.keys():
+            tensors[name] = f.get_tensor(name)
+    return cfg, tensors

@@ -15,7 +15,7 @@ namespace {
 
 constexpr int kWavesPerBlock = 4;
 constexpr int kMaxHeadDim = 256;   // of the values: a lane adds up kMaxHeadDim / 64 channels of the output
-constexpr int kMaxKeyDim = 512;    // of queries and keys, which only enter the scores
+constexpr int kMaxKeyDim = 1024;    // of queries and keys, which only enter the scores
 constexpr int kChanPerLane = kMaxHeadDim / kWave;
 constexpr int kTileMinTokens = 32;  // steps with at least this many tokens share keys and values through LDS
 

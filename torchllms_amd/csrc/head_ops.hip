@@ -20,7 +20,7 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 // Queries go back in place; keys and values go to their pages [page][Hkv][P][dk] and [..][dv] at
 // slot_mapping[t] (keys in place too when there are no pages).
 constexpr int kPrepWaves = 4;
-constexpr int kPrepChan = 8;  // channels a lane holds: heads of up to 512
+constexpr int kPrepChan = 16;  // channels a lane holds: heads of up to 1,024
 
 template <typename T>
 struct PrepArgs {

@@ -31,17 +31,18 @@ def paged_attention(
     sinks=None,
     v_head_dim=None,
     values_in_keys: bool = False,
+    value_offset: int = 0,
 ) -> torch.Tensor:
     """Attention of this step's queries (first Hq * dh columns of ``qkv``) over their requests'
     cached keys and values; returns [n_tokens, Hq * dv].  Capped scores (``softcap``), chunks
     (``chunk``) and sinks are every kernel's; values of another head size than the keys, or values that are
-    the first channels of the key rows (``values_in_keys``), are the plain kernel's alone."""
+    channels of the key rows (``values_in_keys``, from ``value_offset`` on), are the plain kernel's alone."""
     n = qkv.shape[0]
     n_dec = ctx.host.n_decode
     v_dim = head_dim if v_head_dim is None else int(v_head_dim)
     plain_only = v_dim != head_dim or values_in_keys  # (the MFMA kernels take a cap, chunks and sinks, but one head size)
     extended = softcap > 0 or chunk > 0 or sinks is not None or plain_only
-    extras = dict(softcap=softcap, chunk=chunk, sinks=sinks, v_head_dim=v_dim, values_in_keys=values_in_keys) if extended else {}
+    extras = dict(softcap=softcap, chunk=chunk, sinks=sinks, v_head_dim=v_dim, values_in_keys=values_in_keys, value_offset=value_offset) if extended else {}
     fast_extras = dict(softcap=softcap, chunk=chunk, sinks=sinks) if extended else {}
     fast_decode = not plain_only and n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
     # the MFMA prefill kernel takes positive softmax scales only; anything else runs the plain kernel

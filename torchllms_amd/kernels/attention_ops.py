@@ -29,17 +29,19 @@ from .base import (  # noqa: F401
 #: ``DECODE_HEAD_DIMS`` / ``PREFILL_HEAD_DIMS``, everything else below this runs the plain kernel)
 ATTENTION_MAX_HEAD_DIM = 256
 #: the largest head size of queries and keys that the plain kernel takes (they only enter the scores)
-ATTENTION_MAX_KEY_DIM = 512
+ATTENTION_MAX_KEY_DIM = 1024
 
 
 def _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq, positions, block_table, out,
-                       sinks=None, v_head_dim=None, values_in_keys=False):
+                       sinks=None, v_head_dim=None, values_in_keys=False, value_offset=0):
     """What both launches of the plain kernel ask of their arguments; returns (tokens, page size, out, value head
     size, elements between two value rows).  ``values_in_keys``: a token's value is the first ``v_head_dim`` channels
-    of its key row, and ``v_pages`` is ``k_pages``."""
+    of its key row, and ``v_pages`` is ``k_pages``; ``value_offset``: it is the ``v_head_dim`` channels from there on."""
     v_dim = head_dim if v_head_dim is None else int(v_head_dim)
-    if values_in_keys and (v_pages.data_ptr() != k_pages.data_ptr() or v_pages.shape != k_pages.shape or v_dim > head_dim):
-        raise KernelError("attention: values inside the keys are the keys' own pages and at most as wide")
+    if values_in_keys and (v_pages.data_ptr() != k_pages.data_ptr() or v_pages.shape != k_pages.shape or value_offset < 0 or value_offset + v_dim > head_dim):
+        raise KernelError("attention: values inside the keys are the keys' own pages and lie inside the key rows")
+    if value_offset and not values_in_keys:
+        raise KernelError("attention: value_offset is for values inside the keys")
     if sinks is not None and (not sinks.is_cuda or sinks.dtype != torch.float32 or sinks.numel() != n_q_heads or not sinks.is_contiguous()):
         raise KernelError(f"attention: sinks must be a contiguous float32 GPU vector of {n_q_heads} entries")
     _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
@@ -83,18 +85,20 @@ def attention_generic(
     sinks: Optional[torch.Tensor] = None,
     v_head_dim: Optional[int] = None,
     values_in_keys: bool = False,
+    value_offset: int = 0,
 ) -> torch.Tensor:
     """Attention of each token's query heads (the first Hq * dh columns of ``qkv``) over the paged
     keys and values of its request; returns [n, Hq * dv].  ``softcap`` c > 0: scores become
     c * tanh(score / c).  ``chunk`` > 0: a query sees only the keys of its own chunk of that many
     positions.  ``sinks``: one 32-bit number per query head whose exponential joins the softmax's
     denominator.  ``v_head_dim``: the values' head size when it is not the keys'.  ``values_in_keys``: a
-    token's value is the first ``v_head_dim`` channels of its key row (``v_pages`` is ``k_pages``)."""
+    token's value is ``v_head_dim`` channels of its key row, from ``value_offset`` on (``v_pages`` is ``k_pages``)."""
     n, page_size, out, v_dim, v_pitch = _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq,
-                                                           positions, block_table, out, sinks, v_head_dim, values_in_keys)
+                                                           positions, block_table, out, sinks, v_head_dim, values_in_keys, value_offset)
+    v_at = v_pages.data_ptr() + int(value_offset) * v_pages.element_size()
     check(
         core().tl_attention_generic(
-            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_at,
             token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
             n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), float(softcap), int(chunk), _ptr(sinks), v_dim,
             v_pitch, dtype_code(qkv.dtype), _stream(),
@@ -124,19 +128,21 @@ def attention_generic_split(
     sinks: Optional[torch.Tensor] = None,
     v_head_dim: Optional[int] = None,
     values_in_keys: bool = False,
+    value_offset: int = 0,
 ) -> torch.Tensor:
     """``attention_generic`` for steps with few tokens and long contexts (decode): every block of 64
     keys is computed by a wave of its own and a second kernel joins the blocks in order.  The same
     blocks, operations and order as the one-wave form: the same bits.  ``longest``: an upper bound of
     the keys any token sees (its position + 1, or the window)."""
     n, page_size, out, v_dim, v_pitch = _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq,
-                                                           positions, block_table, out, sinks, v_head_dim, values_in_keys)
+                                                           positions, block_table, out, sinks, v_head_dim, values_in_keys, value_offset)
+    v_at = v_pages.data_ptr() + int(value_offset) * v_pages.element_size()
     # blocks are aligned to absolute positions: a range of `longest` keys touches at most this many
     max_blocks = max(int(longest), 1) // 64 + 2
     partials = torch.empty((n, n_q_heads, max_blocks, v_dim + 2), dtype=torch.float32, device=qkv.device)
     check(
         core().tl_attention_generic_split(
-            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
+            qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_at,
             token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
             n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), float(softcap), int(chunk), _ptr(sinks), v_dim,
             v_pitch, dtype_code(qkv.dtype), max_blocks, partials.data_ptr(), _stream(),

@@ -12,8 +12,8 @@ import torch
 
 from .base import KernelError, _gpu, _i32, _ptr, _stream, check, core, dtype_code
 
-#: the widest head ``head_prepare`` takes (eight channels a lane)
-HEAD_PREPARE_MAX_DIM = 512
+#: the widest head ``head_prepare`` takes (sixteen channels a lane)
+HEAD_PREPARE_MAX_DIM = 1024
 
 
 def _f32_vector(v: Optional[torch.Tensor], n: int, what: str) -> None:

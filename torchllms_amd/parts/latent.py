@@ -88,8 +88,6 @@ class LatentAttention(Mixer):
         return specs
 
     def check_sizes(self, dtype: torch.dtype) -> None:
-        if not 0 < self.kv_rank <= ops.ATTENTION_MAX_HEAD_DIM:
-            raise ValueError(f"latent attention: a latent of {self.kv_rank} channels; the attention kernel takes values of up to {ops.ATTENTION_MAX_HEAD_DIM}")
         if self.key_dim > min(ops.ATTENTION_MAX_KEY_DIM, ops.HEAD_PREPARE_MAX_DIM):
             raise ValueError(f"latent attention: rows of {self.key_dim} channels (latent and rotated part); the kernels take "
                              f"{min(ops.ATTENTION_MAX_KEY_DIM, ops.HEAD_PREPARE_MAX_DIM)}")
@@ -154,10 +152,15 @@ class LatentAttention(Mixer):
             ops.head_prepare(q, H, 0, d + r, 0, cos_sin=table, rot_offset=d, rot_dims=r, pairing=pairing)
         q_lat = self._per_head(q.view(n, H, d + r)[:, :, :d], self.w_uk_t)       # [H, n, R]
         queries = ops.pack_heads(q_lat, q, d + r, d, r)                           # [n, H * (R + r)]
-        mixed = paged_attention(
-            queries, H, 1, R + r, cache.k_pages, cache.v_pages, ctx, g, 0, self.softmax_scale, v_head_dim=R, values_in_keys=True,
-        )                                                                         # [n, H * R]: the heads' mixed latents
-        heads = self._per_head(mixed.view(n, H, R), self.w_uv)                    # [H, n, dv]
+        # the heads' mixed latents [n, H, R]; a latent wider than the attention kernel's values is mixed in pieces
+        piece = ops.ATTENTION_MAX_HEAD_DIM
+        parts = [
+            paged_attention(queries, H, 1, R + r, cache.k_pages, cache.v_pages, ctx, g, 0, self.softmax_scale,
+                            v_head_dim=min(piece, R - at), values_in_keys=True, value_offset=at).view(n, H, -1)
+            for at in range(0, R, piece)
+        ]
+        mixed = parts[0] if len(parts) == 1 else torch.cat(parts, dim=2)
+        heads = self._per_head(mixed, self.w_uv)                                  # [H, n, dv]
         gates = down[:, self.q_rank + R + r :] if self.head_gate else None
         out = ops.unpack_heads_gate(heads.contiguous(), gates)
         return ops.linear_to_sum(out, self.wo, may_wait=True)
