@@ -2,7 +2,7 @@
 bfloat16 weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
-                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products|taluvik]
+                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products|taluvik|vobolorn]
 
 Everything runs through the generation loop: the scheduler admits the requests, cuts their prompts
 into portions under its token budget, and plans every decode step; the step function runs it; the
@@ -29,7 +29,8 @@ library's large matrix product.  ``--workload small-kernels`` times what a norm 
 replayed graph of large products, without a profiler (under rocprofv3 no dispatch is shorter than
 about 4.6 us, an empty kernel included, so a kernel trace overstates the small kernels of a step).
 ``--workload taluvik``: prefill and decode of a Taluvik model (chunked attention with sinks, gated delta
-rule, selective scan) beside a Llama model of the same layer sizes.  ``--workload attention``: the decode attention and the merge of its splits alone, by batch size, context and
+rule, selective scan) beside a Llama model of the same layer sizes.  ``--workload vobolorn``: the same for a Vobolorn model (grouped-query layers with normed heads, a query factor, mixed
+values and gates, and attention through a latent, over a 32-bit stream).  ``--workload attention``: the decode attention and the merge of its splits alone, by batch size, context and
 split size.  ``--workload products``: a decode layer's four products alone at 1 to 128 rows, the library against
 this package's kernels.  Both as a step runs them: in a replayed graph, caches flushed.
 """
@@ -83,8 +84,8 @@ def parse_args(argv=None):
     p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the headline's)")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products", "taluvik"])
-    p.add_argument("--only", default=None, choices=["taluvik", "llama"], help="taluvik: measure one of the two models only")
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products", "taluvik", "vobolorn"])
+    p.add_argument("--only", default=None, choices=["taluvik", "vobolorn", "llama"], help="taluvik, vobolorn: measure one of the two models only")
     p.add_argument("--token-budget", type=int, default=8192, help="tokens a step may hold (the scheduler cuts prompts to it)")
     p.add_argument("--no-reference-workload", action="store_true",
                    help="leave out the reference's benchmark (2,048-token prompts, 256 new tokens at batch 1, 8, 64)")
@@ -317,22 +318,45 @@ def taluvik_config(shape: dict, n_layers: int, chunk: int) -> dict:
             "layers": [{"type": turn[i % 4], "mixer": mixers[turn[i % 4]], "mlp": ff} for i in range(n_layers)]}
 
 
+def vobolorn_config(shape: dict, n_layers: int) -> dict:
+    """A Vobolorn configuration with the layer sizes of ``shape`` (a Llama configuration): the same width,
+    feed-forward, heads and head size (keys and values alike, so that the matrix-core attention kernels
+    serve the grouped-query layers); the latent layers with a latent of 192 channels and a rotated part of
+    64 (rows of 256 channels, which those kernels take too) and a query latent of 3/8 of the width; the
+    mixers take turns (query factor, query factor, latent, biases and gate)."""
+    D, H, G, dh = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"]
+    ff = {"kind": "dense", "ff": shape["intermediate_size"]}
+    grouped = {"heads": H, "kv_heads": G, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "v_mix": True}
+    mixers = {
+        "attention": grouped,
+        "attention_2": dict(grouped, q_temp={"coef": 0.1, "every": 1024}),
+        "latent_attention": {"heads": H, "dim": dh, "rot_dim": 64, "vdim": dh, "q_rank": 3 * D // 8, "kv_rank": 192,
+                             "scale": (dh + 64) ** -0.5, "rot": {"base": shape["rope_theta"], "dims": 64}},
+    }
+    turn = ["attention_2", "attention_2", "latent_attention", "attention"]
+    return {"architecture": "Vobolorn", "vocab": shape["vocab_size"], "width": D, "norm": {"eps": 1e-5}, "logit_softcap": 30.0,
+            "layers": [{"type": turn[i % 4], "mixer": mixers[turn[i % 4]], "mlp": ff} for i in range(n_layers)]}
+
+
 def taluvik_run(args, shape) -> int:
-    """Prefill and decode of a Taluvik model beside a Llama model of the same layer sizes and number of
-    layers, both with random weights, both through the same engine, scheduler and generation loop:
-    a prompt of ``--prefill-tokens`` in one step (tokens/s), and decode steps of whole batches whose
-    context ends at ``--context`` (ms a step, tokens/s), at ``--batch`` and ``--points``."""
+    """Prefill and decode of a Taluvik (or, ``--workload vobolorn``, a Vobolorn) model beside a Llama model of the
+    same layer sizes and number of layers, both with random weights, both through the same engine, scheduler and
+    generation loop: a prompt of ``--prefill-tokens`` in one step (tokens/s), and decode steps of whole batches
+    whose context ends at ``--context`` (ms a step, tokens/s), at ``--batch`` and ``--points``."""
     import torch
 
     from torchllms_amd.config import LlamaConfig, TaluvikConfig
+    from torchllms_amd.config.vobolorn import VobolornConfig
     from torchllms_amd.engine import Engine
     from torchllms_amd.sampling import Sampler
 
     n_layers = args.layers or 8
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
     pages_per_req = -(-max(args.context, args.prefill_tokens) // args.page_size) + 1
+    design = "Vobolorn" if args.workload == "vobolorn" else "Taluvik"
     configs = {
-        "taluvik": TaluvikConfig.from_dict(taluvik_config(shape, n_layers, chunk=8192)),
+        args.workload: (VobolornConfig.from_dict(vobolorn_config(shape, n_layers)) if args.workload == "vobolorn"
+                        else TaluvikConfig.from_dict(taluvik_config(shape, n_layers, chunk=8192))),
         "llama": LlamaConfig.from_dict(dict(shape, num_hidden_layers=n_layers)),
     }
     if args.only:
@@ -357,11 +381,11 @@ def taluvik_run(args, shape) -> int:
     first = next(iter(out.values()))
     ms = first[f"decode_b{args.batch}"]["ms_per_step"]
     print(json.dumps({
-        "metric": f"decode tok/s, batch {args.batch}, context {args.context}, Taluvik beside Llama at {SHAPE_NAMES[args.shape]} layer sizes, {n_layers} layers",
+        "metric": f"decode tok/s, batch {args.batch}, context {args.context}, {design} beside Llama at {SHAPE_NAMES[args.shape]} layer sizes, {n_layers} layers",
         "value": first[f"decode_b{args.batch}"]["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random-init weights, random token ids",
-        "config": {"model": f"Taluvik and Llama at {SHAPE_NAMES[args.shape]} layer sizes", "global_batch": args.batch, "seq_len": args.context,
+        "config": {"model": f"{design} and Llama at {SHAPE_NAMES[args.shape]} layer sizes", "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single GPU", "n_layers": n_layers, "page_size": args.page_size},
         "models": out,
     }))
@@ -597,7 +621,7 @@ def main(argv=None) -> int:
         return products_run(args, shape)
     if args.workload == "peaks":
         return peaks_run(args)
-    if args.workload == "taluvik":
+    if args.workload in ("taluvik", "vobolorn"):
         return taluvik_run(args, shape)
     import torch
 

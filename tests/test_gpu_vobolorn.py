@@ -140,6 +140,10 @@ ALONE = {
     "latent": [models.layer(models.latent(3, 16, 8, 24, 12, 36, 0.4))],
     "latent_one_head_wide_rotation": [models.layer(models.latent(1, 8, 64, 8, 40, 16, 0.2, base=100.0))],
     "latent_wider_than_the_values_the_kernel_takes": [models.layer(models.latent(2, 16, 4, 16, 16, 260, 0.3))],
+    # latent and rotated part together make rows that the matrix-core attention kernels take (bfloat16 runs those,
+    # twelve heads in two calls at 256 channels)
+    "latent_matrix_cores_256": [models.layer(models.latent(12, 16, 64, 16, 24, 192, 0.2))],
+    "latent_matrix_cores_64": [models.layer(models.latent(5, 24, 16, 8, 20, 48, 0.3))],
     # heads of one size that the matrix-core attention kernels take (bfloat16 runs those)
     "matrix_cores_64": [models.layer(models.grouped("attention", 8, 2, 64, 64, 0.3, v_mix=True)),
                         models.layer(models.grouped("attention_2", 4, 2, 64, 64, 0.3, q_temp=(0.5, 20), v_mix=True))],
@@ -206,7 +210,7 @@ def test_head_prepare_against_its_formulas(dtype, pairing):
     lam = torch.tensor([0.3])
     inv_freq = 1.0 / (50.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot))
     pos = torch.tensor(positions, dtype=torch.int32)
-    ang = pos.double()[:, None] * inv_freq.double()[None, :]
+    ang = (pos.float()[:, None] * inv_freq[None, :]).double()  # (the angle is a 32-bit product, as in the engine)
     page_size, n_pages = 4, 9
     slots = torch.tensor([3, 0, 35, 9, 8, 17, 21, 22, 23, 1, 30, 31, 12, 2], dtype=torch.int32)
 

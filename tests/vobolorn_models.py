@@ -71,8 +71,9 @@ def single_layer(entry: dict, width: int = 64, vocab: int = 61, softcap=None) ->
 
 #: how much a tensor of a mixer is scaled up after the random-weights mode has drawn it from N(0, 0.02) (or from
 #: N(0, 0.02) around zero for biases): projections before a norm need no scale, what stands behind one or enters a
-#: sigmoid does, or a forgotten bias, gate or rotated part would hardly show
-_SCALES = {"mix.q.b": 12.0, "mix.k.b": 12.0, "mix.v.b": 12.0, "mix.g": 12.0, "mix.uq": 20.0, "mix.uk": 20.0, "mix.dkv": 3.0}
+#: sigmoid does, or a forgotten bias, gate or rotated part would hardly show; the output matrix is scaled so that the
+#: logits reach the cap
+_SCALES = {"head": 40.0, "mix.q.b": 12.0, "mix.k.b": 12.0, "mix.v.b": 12.0, "mix.g": 12.0, "mix.uq": 20.0, "mix.uk": 20.0, "mix.dkv": 3.0}
 
 
 def make_folder(path, cfg_dict: dict, seed: int = 0, dtype=torch.bfloat16) -> Path:

@@ -126,6 +126,31 @@ class LatentAttention(Mixer):
             return out
         return torch.bmm(x.transpose(0, 1), w.transpose(1, 2))
 
+    def _mixed_latents(self, queries, n, ctx, cache):
+        """Attention of the packed queries over the cached rows: every head's softmax-weighted sum of the latents,
+        [n, H, kv_rank]."""
+        H, r, R = self.num_heads, self.rot_dim, self.kv_rank
+        g, kd = cache.group, self.key_dim
+        per_call = 8 if kd == 256 else 16  # query heads per kv head that the matrix-core kernels take
+        if (ops.decode_attention_supported(queries.dtype, per_call, 1, kd)
+                and ops.prefill_attention_supported(queries.dtype, per_call, 1, kd, cache.page_size)):
+            # rows of a size that the matrix-core kernels take: they mix whole rows (the rotated part rides along
+            # and is dropped), one kv head for up to per_call query heads at a time
+            outs = []
+            for h0 in range(0, H, per_call):
+                hg = min(per_call, H - h0)
+                outs.append(paged_attention(queries[:, h0 * kd : (h0 + hg) * kd], hg, 1, kd, cache.k_pages, cache.v_pages, ctx, g, 0,
+                                            self.softmax_scale).view(n, hg, kd)[:, :, :R])
+            return outs[0] if len(outs) == 1 else torch.cat(outs, dim=1)
+        # the plain kernel reads the values out of the key rows; a latent wider than its values is mixed in pieces
+        piece = ops.ATTENTION_MAX_HEAD_DIM
+        parts = [
+            paged_attention(queries, H, 1, kd, cache.k_pages, cache.v_pages, ctx, g, 0, self.softmax_scale,
+                            v_head_dim=min(piece, R - at), values_in_keys=True, value_offset=at).view(n, H, -1)
+            for at in range(0, R, piece)
+        ]
+        return parts[0] if len(parts) == 1 else torch.cat(parts, dim=2)
+
     def forward(self, x, ctx, cache):
         H, d, r, R = self.num_heads, self.head_dim, self.rot_dim, self.kv_rank
         g = cache.group
@@ -152,14 +177,7 @@ class LatentAttention(Mixer):
             ops.head_prepare(q, H, 0, d + r, 0, cos_sin=table, rot_offset=d, rot_dims=r, pairing=pairing)
         q_lat = self._per_head(q.view(n, H, d + r)[:, :, :d], self.w_uk_t)       # [H, n, R]
         queries = ops.pack_heads(q_lat, q, d + r, d, r)                           # [n, H * (R + r)]
-        # the heads' mixed latents [n, H, R]; a latent wider than the attention kernel's values is mixed in pieces
-        piece = ops.ATTENTION_MAX_HEAD_DIM
-        parts = [
-            paged_attention(queries, H, 1, R + r, cache.k_pages, cache.v_pages, ctx, g, 0, self.softmax_scale,
-                            v_head_dim=min(piece, R - at), values_in_keys=True, value_offset=at).view(n, H, -1)
-            for at in range(0, R, piece)
-        ]
-        mixed = parts[0] if len(parts) == 1 else torch.cat(parts, dim=2)
+        mixed = self._mixed_latents(queries, n, ctx, cache)                       # [n, H, R]
         heads = self._per_head(mixed, self.w_uv)                                  # [H, n, dv]
         gates = down[:, self.q_rank + R + r :] if self.head_gate else None
         out = ops.unpack_heads_gate(heads.contiguous(), gates)
