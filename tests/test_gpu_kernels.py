@@ -576,8 +576,12 @@ def test_attention_refuses_sizes_it_does_not_have():
 
     q = torch.zeros(1, 2 * 272, device=DEV)
     pages = torch.zeros(2, 2, 4, 272, device=DEV)
-    with pytest.raises(KernelError, match="head_dim=272"):
+    with pytest.raises(KernelError, match="values of head size 272"):
         _ops().attention_generic(q, 2, 2, 272, pages, pages, _i32([0]), _i32([0]), _i32([[0]]), 0, 1.0)
+    q = torch.zeros(1, 2 * 1040, device=DEV)
+    keys, values = torch.zeros(2, 2, 4, 1040, device=DEV), torch.zeros(2, 2, 4, 16, device=DEV)
+    with pytest.raises(KernelError, match="head_dim=1040"):
+        _ops().attention_generic(q, 2, 2, 1040, keys, values, _i32([0]), _i32([0]), _i32([[0]]), 0, 1.0, v_head_dim=16)
     q = torch.zeros(1, 3 * 16, device=DEV)
     pages = torch.zeros(2, 2, 4, 16, device=DEV)
     with pytest.raises(KernelError, match="not a multiple"):

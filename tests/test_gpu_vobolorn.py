@@ -192,7 +192,7 @@ def _bf16_tol(dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("pairing", [0, 1])
 def test_head_prepare_against_its_formulas(dtype, pairing):
-    """Weighted norm over the first channels, rotation of a middle part, the query factor at the positions where
+    """A bias, the weighted norm over the first channels, rotation of a middle part, the query factor at the positions where
     it steps (just below, at and just above multiples of ``every``, and position 0), mixed values, pages."""
     from torchllms_amd.kernels import ops
 
@@ -214,7 +214,10 @@ def test_head_prepare_against_its_formulas(dtype, pairing):
     page_size, n_pages = 4, 9
     slots = torch.tensor([3, 0, 35, 9, 8, 17, 21, 22, 23, 1, 30, 31, 12, 2], dtype=torch.int32)
 
+    heads_width = (H + G) * dk + G * dv
+    bias = torch.randn(heads_width, generator=g).to(dtype)
     x = rows.double()
+    x[:, :heads_width] = (rows[:, :heads_width].float() + bias.float()).to(dtype).double()  # (stored as a projection with a bias would be)
     q = x[:, : H * dk].reshape(n, H, dk).clone()
     k = x[:, H * dk : (H + G) * dk].reshape(n, G, dk).clone()
     v = x[:, (H + G) * dk : (H + G) * dk + G * dv].reshape(n, G, dv)
@@ -244,7 +247,7 @@ def test_head_prepare_against_its_formulas(dtype, pairing):
     k_pages = torch.zeros((n_pages, G, page_size, dk), dtype=dtype, device=dev)
     v_pages = torch.zeros((n_pages, G, page_size, dv), dtype=dtype, device=dev)
     table = ops.rope_table(pos.to(dev), inv_freq.to(dev))
-    ops.head_prepare(d_rows, H, G, dk, dv, q_norm=qw.to(dev), k_norm=kw.to(dev), norm_dims=norm_dims, eps=eps, cos_sin=table,
+    ops.head_prepare(d_rows, H, G, dk, dv, bias=bias.to(dev), q_norm=qw.to(dev), k_norm=kw.to(dev), norm_dims=norm_dims, eps=eps, cos_sin=table,
                      rot_offset=rot_off, rot_dims=rot, pairing=pairing, positions=pos.to(dev), temp_coef=coef, temp_every=every,
                      v_first=v_first.to(dev), v_mix=lam.to(dev), k_pages=k_pages, v_pages=v_pages, slot_mapping=slots.to(dev),
                      page_size=page_size)
@@ -282,15 +285,16 @@ def test_branch_norm_and_the_other_small_kernels(dtype):
     got = ops.rmsnorm_columns(wide.to(dev)[:, 11 : 11 + hidden], w.to(dev), 1e-4, dtype, rows=idx.to(dev))
     sel = part[idx.long()].double()
     torch.testing.assert_close(got.cpu().double(), sel / torch.sqrt((sel ** 2).mean(-1, keepdim=True) + 1e-4) * w.double(), **_bf16_tol(dtype))
-    # gates channel by channel and head by head
+    # gates channel by channel and head by head (sizes that the 16-byte form takes, and sizes that it does not)
+    for heads, d in ((6, 20), (8, 16)):
+        x = torch.randn((n, heads * d), generator=g).to(dtype)
+        gates = torch.randn((n, heads * d + heads), generator=g).to(dtype)
+        by_channel = ops.sigmoid_gate_(x.to(dev).clone(), gates.to(dev)[:, : heads * d], per=1)
+        torch.testing.assert_close(by_channel.cpu().double(), x.double() * torch.sigmoid(gates[:, : heads * d].double()), **_bf16_tol(dtype))
+        by_head = ops.sigmoid_gate_(x.to(dev).clone(), gates.to(dev)[:, heads * d :], per=d)
+        want_h = x.double().reshape(n, heads, d) * torch.sigmoid(gates[:, heads * d :].double())[:, :, None]
+        torch.testing.assert_close(by_head.cpu().double().reshape(n, heads, d), want_h, **_bf16_tol(dtype))
     heads, d = 6, 20
-    x = torch.randn((n, heads * d), generator=g).to(dtype)
-    gates = torch.randn((n, heads * d + heads), generator=g).to(dtype)
-    by_channel = ops.sigmoid_gate_(x.to(dev).clone(), gates.to(dev)[:, : heads * d], per=1)
-    torch.testing.assert_close(by_channel.cpu().double(), x.double() * torch.sigmoid(gates[:, : heads * d].double()), **_bf16_tol(dtype))
-    by_head = ops.sigmoid_gate_(x.to(dev).clone(), gates.to(dev)[:, heads * d :], per=d)
-    want_h = x.double().reshape(n, heads, d) * torch.sigmoid(gates[:, heads * d :].double())[:, :, None]
-    torch.testing.assert_close(by_head.cpu().double().reshape(n, heads, d), want_h, **_bf16_tol(dtype))
     # packing and unpacking of heads
     a = torch.randn((heads, n, 9), generator=g).to(dtype)
     b = torch.randn((n, heads * 14 + 3), generator=g).to(dtype)

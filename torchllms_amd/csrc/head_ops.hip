@@ -12,6 +12,7 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 // ----------------------------------------------------------------------------- heads before the scores
 // rows: [n_tokens, row_stride], a row = Hq query heads of dk | Hkv key heads of dk | Hkv value heads of dv |
 // whatever follows (left alone).  One wave a head:
+//   every head first takes its bias (bias given: one entry per column of the heads, q | k | v);
 //   query and key heads: the first norm_dims channels become x / sqrt(mean(x^2) + eps) * w (w given; q_w for
 //     queries, k_w for keys), the channels rot_off .. rot_off + rot - 1 are rotated by the step's table of
 //     cosines and sines (pairing 0: (2i, 2i+1); 1: (i, i + rot/2)), queries are multiplied by
@@ -20,12 +21,13 @@ __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf
 // Queries go back in place; keys and values go to their pages [page][Hkv][P][dk] and [..][dv] at
 // slot_mapping[t] (keys in place too when there are no pages).
 constexpr int kPrepWaves = 4;
-constexpr int kPrepChan = 16;  // channels a lane holds: heads of up to 1,024
+constexpr int kPrepMaxChan = 16;  // channels a lane holds at most: heads of up to 1,024
 
 template <typename T>
 struct PrepArgs {
   T* rows;
   int row_stride, n_q, n_kv, dk, dv;
+  const T* bias;
   const float* q_w;
   const float* k_w;
   int norm_dims;
@@ -44,7 +46,8 @@ struct PrepArgs {
   int page_size;
 };
 
-template <typename T>
+// kPrepChan: channels a lane holds (the widest head of the launch over 64, rounded up to a power of two).
+template <typename T, int kPrepChan>
 __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const PrepArgs<T> a) {
   __shared__ float turned[kPrepWaves][kPrepChan * kWave];
   const int t = blockIdx.x;
@@ -65,10 +68,13 @@ __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const P
                  : base + (size_t)(live ? unit : 0) * a.dk;
   float val[kPrepChan];
   float ss = 0.f;
+  const T* head_bias = a.bias ? a.bias + (head - base) : nullptr;
 #pragma unroll
   for (int c = 0; c < kPrepChan; ++c) {
     const int d = lane + c * kWave;
     val[c] = (live && d < width) ? to_f32(head[d]) : 0.f;
+    // (the sum is rounded to the rows' type, as a projection with a bias would have stored it)
+    if (head_bias && live && d < width) val[c] = to_f32(from_f32<T>(val[c] + to_f32(head_bias[d])));
     if (d < a.norm_dims) ss += val[c] * val[c];
   }
   const float* w = is_q ? a.q_w : (is_k ? a.k_w : nullptr);
@@ -83,9 +89,11 @@ __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const P
   }
   // rotation: every lane needs its partner's channel as it is after the norm
   const bool turns = (is_q || is_k) && a.rot > 0;
+  if (a.rot > 0) {  // (uniform over the block)
 #pragma unroll
-  for (int c = 0; c < kPrepChan; ++c) turned[wave][lane + c * kWave] = val[c];
-  __syncthreads();
+    for (int c = 0; c < kPrepChan; ++c) turned[wave][lane + c * kWave] = val[c];
+    __syncthreads();
+  }
   if (turns) {
     const int rh = a.rot / 2;
 #pragma unroll
@@ -129,6 +137,13 @@ __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const P
   }
   // a value head
   const int g = unit - a.n_q - a.n_kv;
+  if (a.v_first == nullptr && a.bias != nullptr) {  // (values with a bias and no mixing go back too: later layers may read them)
+#pragma unroll
+    for (int c = 0; c < kPrepChan; ++c) {
+      const int d = lane + c * kWave;
+      if (d < width) head[d] = from_f32<T>(val[c]);
+    }
+  }
   if (a.v_first != nullptr) {
     const float lam = a.lam[0];
     const T* vf = a.v_first + (size_t)t * a.v_first_stride + (size_t)g * a.dv;
@@ -155,6 +170,50 @@ __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const P
 // stream[r, :] += y[r, :] / sqrt(mean(y[r, :]^2) + eps) * w   (32-bit), and rows[r, :] = T(stream[r, :]) for the
 // next reader (rows may be null).  A block a row; the statistics in a fixed order.
 constexpr int kRowThreads = 256;
+constexpr int kRowHeldMost = 32;  // elements a thread holds at most in the form that reads everything at once: rows of up to 8,192
+
+// The same for rows that the block's registers hold: the branch, the stream and the weight are all asked for before
+// anything waits, so a row costs one trip to memory and not three (a step of few rows is nothing but that wait).
+// The sums are those of the kernel below, in the same order.
+template <typename T, int kRowHeld>
+__global__ void __launch_bounds__(kRowThreads)
+branch_norm_add_held_kernel(float* __restrict__ stream, const T* __restrict__ y, const float* __restrict__ w,
+                            T* __restrict__ rows, int hidden, float eps) {
+  __shared__ float scratch[kRowThreads / kWave];
+  const size_t r = blockIdx.x;
+  const T* yr = y + r * hidden;
+  float* sr = stream + r * hidden;
+  // every load is made whatever the row's width (an element past the end is the row's first once more, and not
+  // used): a select right behind a load makes the wave wait for each load in turn
+  T yraw[kRowHeld];
+  float sv[kRowHeld], wv[kRowHeld];
+#pragma unroll
+  for (int c = 0; c < kRowHeld; ++c) {
+    const int i = threadIdx.x + c * kRowThreads;
+    const int at = i < hidden ? i : 0;
+    yraw[c] = yr[at];
+    sv[c] = sr[at];
+    wv[c] = w[at];
+  }
+  float yv[kRowHeld];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < kRowHeld; ++c) {
+    yv[c] = threadIdx.x + c * kRowThreads < hidden ? to_f32(yraw[c]) : 0.f;
+    ss += yv[c] * yv[c];
+  }
+  ss = block_sum<kRowThreads / kWave>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+#pragma unroll
+  for (int c = 0; c < kRowHeld; ++c) {
+    const int i = threadIdx.x + c * kRowThreads;
+    if (i < hidden) {
+      const float h = sv[c] + yv[c] * inv * wv[c];
+      sr[i] = h;
+      if (rows) rows[r * hidden + i] = from_f32<T>(h);
+    }
+  }
+}
 
 template <typename T>
 __global__ void __launch_bounds__(kRowThreads)
@@ -188,14 +247,35 @@ rmsnorm_columns_kernel(const XT* __restrict__ x, int x_stride, const int32_t* __
   const size_t r = blockIdx.x;
   const size_t s = rows ? (size_t)rows[r] : r;
   const XT* xr = x + s * x_stride;
+  // eight loads are asked for together, whatever the width (an element past the end is the first once more, and
+  // not used); the sums keep the order of one element after the other
+  constexpr int U = 8;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += kRowThreads) {
-    const float v = to_f32(xr[i]);
-    ss += v * v;
+  for (int i0 = threadIdx.x; i0 < width; i0 += U * kRowThreads) {
+    XT raw[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) raw[u] = xr[i0 + u * kRowThreads < width ? i0 + u * kRowThreads : 0];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float v = i0 + u * kRowThreads < width ? to_f32(raw[u]) : 0.f;
+      ss += v * v;
+    }
   }
   ss = block_sum<kRowThreads / kWave>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  for (int i = threadIdx.x; i < width; i += kRowThreads) y[r * y_stride + i] = from_f32<T>(to_f32(xr[i]) * inv * w[i]);
+  for (int i0 = threadIdx.x; i0 < width; i0 += U * kRowThreads) {
+    XT raw[U];
+    float wv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int at = i0 + u * kRowThreads < width ? i0 + u * kRowThreads : 0;
+      raw[u] = xr[at];
+      wv[u] = w[at];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (i0 + u * kRowThreads < width) y[r * y_stride + i0 + u * kRowThreads] = from_f32<T>(to_f32(raw[u]) * inv * wv[u]);
+  }
 }
 
 // ----------------------------------------------------------------------------- gates, packing, cap
@@ -210,6 +290,42 @@ __global__ void sigmoid_gate_kernel(T* __restrict__ x, int x_stride, const T* __
     const int c = (int)(idx % width);
     T* p = x + t * x_stride + c;
     *p = from_f32<T>(to_f32(*p) * sigmoid_f(to_f32(g[t * g_stride + c / per])));
+  }
+}
+
+// The same for bfloat16 rows whose eight-element pieces are aligned: a thread takes 16 bytes of x (and of the gates,
+// channel by channel; head by head the eight channels share one gate).
+__global__ void sigmoid_gate_wide_kernel(bf16_t* __restrict__ x, int x_stride, const bf16_t* __restrict__ g, int g_stride,
+                                         int n, int width, int per) {
+  const int pieces = width / 8;
+  const size_t total = (size_t)n * pieces;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / pieces;
+    const int c = (int)(idx % pieces) * 8;
+    uint4* p = reinterpret_cast<uint4*>(x + t * x_stride + c);
+    uint4 xv = *p;
+    float gates[8];
+    if (per == 1) {
+      const uint4 gv = *reinterpret_cast<const uint4*>(g + t * g_stride + c);
+      const uint32_t gw[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        gates[2 * e] = sigmoid_f(__uint_as_float(gw[e] << 16));
+        gates[2 * e + 1] = sigmoid_f(__uint_as_float(gw[e] & 0xffff0000u));
+      }
+    } else {
+      const float one = sigmoid_f(to_f32(g[t * g_stride + c / per]));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) gates[e] = one;
+    }
+    uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bf16_t lo = from_f32<bf16_t>(__uint_as_float(xw[e] << 16) * gates[2 * e]);
+      const bf16_t hi = from_f32<bf16_t>(__uint_as_float(xw[e] & 0xffff0000u) * gates[2 * e + 1]);
+      xw[e] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+    }
+    *p = uint4{xw[0], xw[1], xw[2], xw[3]};
   }
 }
 
@@ -248,15 +364,15 @@ int elementwise_blocks(size_t total) {
 
 }  // namespace
 
-TL_EXPORT int tl_head_prepare(void* rows, int row_stride, int n_tokens, int n_q, int n_kv, int dk, int dv,
+TL_EXPORT int tl_head_prepare(void* rows, int row_stride, int n_tokens, int n_q, int n_kv, int dk, int dv, const void* bias,
                               const float* q_w, const float* k_w, int norm_dims, float eps, const float* cos_sin,
                               int rot_off, int rot, int pairing, const int32_t* positions, float temp_coef,
                               int temp_every, const void* v_first, int v_first_stride, const float* lam,
                               void* k_pages, void* v_pages, const int32_t* slot_mapping, int page_size, int dtype,
                               hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q >= 0 && n_kv >= 0 && n_q + n_kv > 0 && dk > 0 && dv >= 0, "head_prepare: bad sizes");
-  TL_REQUIRE(dk <= kPrepChan * kWave && dv <= kPrepChan * kWave, "head_prepare: heads of %d and %d channels, at most %d", dk, dv,
-             kPrepChan * kWave);
+  TL_REQUIRE(dk <= kPrepMaxChan * kWave && dv <= kPrepMaxChan * kWave, "head_prepare: heads of %d and %d channels, at most %d", dk, dv,
+             kPrepMaxChan * kWave);
   TL_REQUIRE(row_stride >= (n_q + n_kv) * dk + n_kv * dv, "head_prepare: rows of %d elements do not hold the heads", row_stride);
   TL_REQUIRE(norm_dims >= 0 && norm_dims <= dk, "head_prepare: a norm over %d of %d channels", norm_dims, dk);
   TL_REQUIRE((q_w == nullptr && k_w == nullptr) || norm_dims > 0, "head_prepare: norm weights without channels to norm");
@@ -269,12 +385,17 @@ TL_EXPORT int tl_head_prepare(void* rows, int row_stride, int n_tokens, int n_q,
   if (n_tokens == 0) return TL_OK;
   const int units = n_q + n_kv + (dv > 0 ? n_kv : 0);
   const dim3 grid(n_tokens, (units + kPrepWaves - 1) / kPrepWaves);
+  const int widest = dk > dv ? dk : dv;
 #define TL_PREP(T)                                                                                                   \
   do {                                                                                                               \
-    PrepArgs<T> a{(T*)rows, row_stride, n_q, n_kv, dk, dv, q_w, k_w, (q_w || k_w) ? norm_dims : 0, eps,              \
+    PrepArgs<T> a{(T*)rows, row_stride, n_q, n_kv, dk, dv, (const T*)bias, q_w, k_w, (q_w || k_w) ? norm_dims : 0, eps,              \
                   (const float2*)cos_sin, rot_off, rot, pairing, positions, temp_coef, temp_every, (const T*)v_first, \
                   v_first_stride, lam, (T*)k_pages, (T*)v_pages, slot_mapping, page_size};                           \
-    head_prepare_kernel<T><<<grid, kPrepWaves * kWave, 0, stream>>>(a);                                              \
+    if (widest <= kWave) head_prepare_kernel<T, 1><<<grid, kPrepWaves * kWave, 0, stream>>>(a);                      \
+    else if (widest <= 2 * kWave) head_prepare_kernel<T, 2><<<grid, kPrepWaves * kWave, 0, stream>>>(a);             \
+    else if (widest <= 4 * kWave) head_prepare_kernel<T, 4><<<grid, kPrepWaves * kWave, 0, stream>>>(a);             \
+    else if (widest <= 8 * kWave) head_prepare_kernel<T, 8><<<grid, kPrepWaves * kWave, 0, stream>>>(a);             \
+    else head_prepare_kernel<T, kPrepMaxChan><<<grid, kPrepWaves * kWave, 0, stream>>>(a);                           \
   } while (0)
   if (dtype == TL_F32) TL_PREP(float);
   else if (dtype == TL_BF16) TL_PREP(bf16_t);
@@ -287,9 +408,21 @@ TL_EXPORT int tl_branch_norm_add(float* stream_rows, const void* y, const float*
                                  int dtype, hipStream_t stream) {
   TL_REQUIRE(n >= 0 && hidden > 0, "branch_norm_add: bad sizes");
   if (n == 0) return TL_OK;
-  if (dtype == TL_F32) branch_norm_add_kernel<float><<<n, kRowThreads, 0, stream>>>(stream_rows, (const float*)y, w, (float*)rows, hidden, eps);
-  else if (dtype == TL_BF16) branch_norm_add_kernel<bf16_t><<<n, kRowThreads, 0, stream>>>(stream_rows, (const bf16_t*)y, w, (bf16_t*)rows, hidden, eps);
+  // few rows: a launch is as long as a row's trips to memory, so everything is fetched at once; many rows hide
+  // the trips behind each other and do better with few registers
+  const bool held = hidden <= kRowHeldMost * kRowThreads && n <= 2 * tl_device_facts().compute_units;
+#define TL_BRANCH(T)                                                                                                              \
+  do {                                                                                                                            \
+    if (!held) branch_norm_add_kernel<T><<<n, kRowThreads, 0, stream>>>(stream_rows, (const T*)y, w, (T*)rows, hidden, eps);      \
+    else if (hidden <= 2 * kRowThreads) branch_norm_add_held_kernel<T, 2><<<n, kRowThreads, 0, stream>>>(stream_rows, (const T*)y, w, (T*)rows, hidden, eps);   \
+    else if (hidden <= 8 * kRowThreads) branch_norm_add_held_kernel<T, 8><<<n, kRowThreads, 0, stream>>>(stream_rows, (const T*)y, w, (T*)rows, hidden, eps);   \
+    else if (hidden <= 16 * kRowThreads) branch_norm_add_held_kernel<T, 16><<<n, kRowThreads, 0, stream>>>(stream_rows, (const T*)y, w, (T*)rows, hidden, eps); \
+    else branch_norm_add_held_kernel<T, kRowHeldMost><<<n, kRowThreads, 0, stream>>>(stream_rows, (const T*)y, w, (T*)rows, hidden, eps);                     \
+  } while (0)
+  if (dtype == TL_F32) TL_BRANCH(float);
+  else if (dtype == TL_BF16) TL_BRANCH(bf16_t);
   else return tl_fail(TL_ERR_ARG, "branch_norm_add: unknown dtype %d", dtype);
+#undef TL_BRANCH
   return tl_check_launch("branch_norm_add");
 }
 
@@ -312,8 +445,14 @@ TL_EXPORT int tl_sigmoid_gate(void* x, int x_stride, const void* g, int g_stride
   if (n == 0) return TL_OK;
   const int blocks = elementwise_blocks((size_t)n * width);
   if (dtype == TL_F32) sigmoid_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, x_stride, (const float*)g, g_stride, n, width, per);
-  else if (dtype == TL_BF16) sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, x_stride, (const bf16_t*)g, g_stride, n, width, per);
-  else return tl_fail(TL_ERR_ARG, "sigmoid_gate: unknown dtype %d", dtype);
+  else if (dtype == TL_BF16) {
+    const bool wide = width % 8 == 0 && x_stride % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
+                      (per == 1 ? (g_stride % 8 == 0 && ((uintptr_t)g % 16) == 0) : per % 8 == 0);
+    if (wide) sigmoid_gate_wide_kernel<<<elementwise_blocks((size_t)n * (width / 8)), 256, 0, stream>>>((bf16_t*)x, x_stride, (const bf16_t*)g, g_stride, n, width, per);
+    else sigmoid_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, x_stride, (const bf16_t*)g, g_stride, n, width, per);
+  } else {
+    return tl_fail(TL_ERR_ARG, "sigmoid_gate: unknown dtype %d", dtype);
+  }
   return tl_check_launch("sigmoid_gate");
 }
 

@@ -27,6 +27,7 @@ def head_prepare(
     n_kv_heads: int,
     head_dim: int,
     v_head_dim: int,
+    bias: Optional[torch.Tensor] = None,
     q_norm: Optional[torch.Tensor] = None,
     k_norm: Optional[torch.Tensor] = None,
     norm_dims: int = 0,
@@ -48,6 +49,7 @@ def head_prepare(
     """Prepare the heads of ``rows`` [n, >= (Hq + Hkv) * dk + Hkv * dv] = query heads | key heads | value
     heads | anything else, in place and into the cache:
 
+    * every head first takes its ``bias`` (one entry per column of the heads, in the rows' dtype; None: none);
     * query and key heads: the first ``norm_dims`` channels are divided by their root mean square
       (``eps`` under the root) and multiplied by ``q_norm`` / ``k_norm`` (32-bit vectors; None: no norm);
       then channels ``rot_offset .. rot_offset + rot_dims`` are rotated by ``cos_sin`` (the step's table);
@@ -56,13 +58,15 @@ def head_prepare(
       and ``v_mix`` (a 32-bit scalar on the device) they become ``(1 - v_mix) v + v_mix v_first``;
     * queries and mixed values are written back, keys and values go to their pages at ``slot_mapping``
       (keys back in place when there are no pages)."""
-    _gpu(rows, q_norm, k_norm, cos_sin, positions, v_first, v_mix, k_pages, v_pages, slot_mapping)
+    _gpu(rows, bias, q_norm, k_norm, cos_sin, positions, v_first, v_mix, k_pages, v_pages, slot_mapping)
     _i32(positions, "positions")
     _i32(slot_mapping, "slot_mapping")
     n = rows.shape[0]
     width = (n_q_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim
     if rows.dim() != 2 or rows.stride(1) != 1 or rows.shape[1] < width:
         raise KernelError(f"head_prepare: rows must be row-major with at least {width} columns, got {tuple(rows.shape)}")
+    if bias is not None and (bias.dim() != 1 or bias.numel() != width or bias.dtype != rows.dtype or not bias.is_contiguous()):
+        raise KernelError(f"head_prepare: bias must be a contiguous vector of {width} entries of the rows' dtype")
     if q_norm is not None or k_norm is not None:
         _f32_vector(q_norm, norm_dims, "head_prepare: q_norm")
         _f32_vector(k_norm, norm_dims, "head_prepare: k_norm")
@@ -87,7 +91,7 @@ def head_prepare(
                 raise KernelError(f"head_prepare: pages must be contiguous [pages, {n_kv_heads}, {page_size}, {d}] of {rows.dtype}")
     check(
         core().tl_head_prepare(
-            rows.data_ptr(), rows.stride(0), n, n_q_heads, n_kv_heads, head_dim, v_head_dim, _ptr(q_norm), _ptr(k_norm),
+            rows.data_ptr(), rows.stride(0), n, n_q_heads, n_kv_heads, head_dim, v_head_dim, _ptr(bias), _ptr(q_norm), _ptr(k_norm),
             int(norm_dims), float(eps), _ptr(cos_sin), int(rot_offset), int(rot_dims), int(pairing), _ptr(positions),
             float(temp_coef), int(temp_every), _ptr(v_first), vf_stride, _ptr(v_mix), _ptr(k_pages),
             _ptr(v_pages) if v_head_dim > 0 else None, _ptr(slot_mapping), int(page_size), dtype_code(rows.dtype), _stream(),

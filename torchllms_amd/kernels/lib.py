@@ -41,7 +41,7 @@ _CORE_SIGNATURES = {
     "tl_causal_conv": [_P, _I, _P, _P, _P, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "tl_selective_scan": [_P, _P, _I, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P],
     "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
-    "tl_head_prepare": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _I, _I, _I, _P, _F, _I, _P, _I, _P, _P, _P, _P, _I, _I, _P],
+    "tl_head_prepare": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _F, _P, _I, _I, _I, _P, _F, _I, _P, _I, _P, _P, _P, _P, _I, _I, _P],
     "tl_branch_norm_add": [_P, _P, _P, _P, _I, _I, _F, _I, _P],
     "tl_rmsnorm_columns": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _F, _P],
     "tl_sigmoid_gate": [_P, _I, _P, _I, _I, _I, _I, _I, _P],

@@ -272,8 +272,6 @@ class Attention(Mixer):
         g = cache.group
         H, dk, dv = self.num_heads, self.head_dim, self.v_head_dim
         rows = ops.linear(ops.resolved(x), self.wqkv)
-        if self.bqkv is not None:
-            ops.add_bias_(rows, self.bqkv)
         v_at = (H + n_kv_in_row) * dk
         v_first = None
         if self.value_mix == "mix":
@@ -281,7 +279,7 @@ class Attention(Mixer):
             if v_first is None:
                 raise RuntimeError(f"attention: no earlier layer of this step has left values under {self.value_mix_key!r}")
         ops.head_prepare(
-            rows, H, n_kv_in_row, dk, dv if n_kv_in_row else 0,
+            rows, H, n_kv_in_row, dk, dv if n_kv_in_row else 0, bias=self.bqkv,
             q_norm=self.q_norm, k_norm=self.k_norm if n_kv_in_row else None, norm_dims=dk if self.qk_norm_weight else 0,
             eps=self.qk_norm_eps, cos_sin=table, rot_offset=0, rot_dims=rot.rotary_dim if rot else 0,
             pairing=rot.pairing if rot else 0, positions=ctx.positions, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every,
