@@ -138,6 +138,7 @@ ALONE = {
                      models.layer(models.grouped("attention", 6, 1, 8, 24, 0.9, v_mix=True)),
                      models.layer(models.grouped("attention_2", 1, 1, 32, 24, 0.4, q_temp=(0.1, 9), v_mix=True))],
     "latent": [models.layer(models.latent(3, 16, 8, 24, 12, 36, 0.4))],
+    "latent_nothing_rotated": [models.layer(models.latent(2, 24, 0, 12, 20, 44, 0.3))],
     "latent_one_head_wide_rotation": [models.layer(models.latent(1, 8, 64, 8, 40, 16, 0.2, base=100.0))],
     "latent_wider_than_the_values_the_kernel_takes": [models.layer(models.latent(2, 16, 4, 16, 16, 260, 0.3))],
     # latent and rotated part together make rows that the matrix-core attention kernels take (bfloat16 runs those,

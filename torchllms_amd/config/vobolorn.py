@@ -102,7 +102,10 @@ class VobolornConfig:
         if lacking:
             raise ConfigError(f"{where}: the {kind} mixer lacks {lacking}")
         for k in _MIXER_KEYS[kind]:
-            if k not in ("scale", "rot"):
+            if k == "rot_dim":  # (a latent layer may rotate nothing)
+                if not isinstance(mixer[k], int) or isinstance(mixer[k], bool) or mixer[k] < 0:
+                    raise ConfigError(f"{where}: rot_dim must be an integer that is not negative, got {mixer[k]!r}")
+            elif k not in ("scale", "rot"):
                 _positive_int(where, k, mixer[k])
         if not _number(where, "scale", mixer["scale"]) > 0:
             raise ConfigError(f"{where}: scale must be positive, got {mixer['scale']!r}")
@@ -160,7 +163,7 @@ def _mixer_spec(cfg: VobolornConfig, i: int) -> PartSpec:
     m = layer.mixer
     if layer.type == "latent_attention":
         position = PartSpec("rope", dict(head_dim=m["rot_dim"], rotary_dim=m["rot_dim"], theta=float(m["rot"]["base"]), scaling=None,
-                                         pairing="interleaved"))
+                                         pairing="interleaved")) if m["rot_dim"] > 0 else PartSpec("none", {})
         return PartSpec("latent_attention", dict(
             hidden_size=cfg.width, num_heads=m["heads"], head_dim=m["dim"], rot_dim=m["rot_dim"], v_head_dim=m["vdim"],
             q_rank=m["q_rank"], kv_rank=m["kv_rank"], softmax_scale=float(m["scale"]), norm_eps=cfg.norm_eps, position=position,

@@ -66,25 +66,37 @@ __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const P
   const int width = is_v ? a.dv : a.dk;
   T* head = is_v ? base + (size_t)(a.n_q + a.n_kv) * a.dk + (size_t)(unit - a.n_q - a.n_kv) * a.dv
                  : base + (size_t)(live ? unit : 0) * a.dk;
-  float val[kPrepChan];
-  float ss = 0.f;
+  // every load is made whatever the head's width (a channel past the end is the head's first once more, and not
+  // used), and nothing looks at a loaded value before all are asked for: a select right behind a load makes the
+  // wave wait for each load in turn
+  const float* w = is_q ? a.q_w : (is_k ? a.k_w : nullptr);
   const T* head_bias = a.bias ? a.bias + (head - base) : nullptr;
+  T raw[kPrepChan], raw_bias[kPrepChan];
+  float wv[kPrepChan];
 #pragma unroll
   for (int c = 0; c < kPrepChan; ++c) {
     const int d = lane + c * kWave;
-    val[c] = (live && d < width) ? to_f32(head[d]) : 0.f;
+    raw[c] = head[d < width ? d : 0];
+    if (head_bias) raw_bias[c] = head_bias[d < width ? d : 0];  // (uniform)
+    if (w) wv[c] = w[d < a.norm_dims ? d : 0];                  // (uniform)
+  }
+  float val[kPrepChan];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < kPrepChan; ++c) {
+    const int d = lane + c * kWave;
+    val[c] = (live && d < width) ? to_f32(raw[c]) : 0.f;
     // (the sum is rounded to the rows' type, as a projection with a bias would have stored it)
-    if (head_bias && live && d < width) val[c] = to_f32(from_f32<T>(val[c] + to_f32(head_bias[d])));
+    if (head_bias && live && d < width) val[c] = to_f32(from_f32<T>(val[c] + to_f32(raw_bias[c])));
     if (d < a.norm_dims) ss += val[c] * val[c];
   }
-  const float* w = is_q ? a.q_w : (is_k ? a.k_w : nullptr);
   if (w != nullptr) {  // (uniform per wave)
     ss = wave_sum(ss);
     const float inv = 1.0f / sqrtf(ss / (float)a.norm_dims + a.eps);
 #pragma unroll
     for (int c = 0; c < kPrepChan; ++c) {
       const int d = lane + c * kWave;
-      if (d < a.norm_dims) val[c] = val[c] * inv * w[d];
+      if (d < a.norm_dims) val[c] = val[c] * inv * wv[c];
     }
   }
   // rotation: every lane needs its partner's channel as it is after the norm
@@ -147,11 +159,14 @@ __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const P
   if (a.v_first != nullptr) {
     const float lam = a.lam[0];
     const T* vf = a.v_first + (size_t)t * a.v_first_stride + (size_t)g * a.dv;
+    T first[kPrepChan];
+#pragma unroll
+    for (int c = 0; c < kPrepChan; ++c) first[c] = vf[lane + c * kWave < width ? lane + c * kWave : 0];
 #pragma unroll
     for (int c = 0; c < kPrepChan; ++c) {
       const int d = lane + c * kWave;
       if (d < width) {
-        val[c] = (1.0f - lam) * val[c] + lam * to_f32(vf[d]);
+        val[c] = (1.0f - lam) * val[c] + lam * to_f32(first[c]);
         head[d] = from_f32<T>(val[c]);
       }
     }
