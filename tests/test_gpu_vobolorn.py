@@ -421,6 +421,42 @@ def test_greedy_generation_through_the_entry_point(tmp_path):
         assert logits[r.token_ids[0]] >= logits.max() - 0.05 * float(logits.std())
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay_program(tmp_path, dtype):
+    """``bin/trace_run`` as a process: steps in, logits files out, the plain model's values; the pool is made for
+    the live requests only, so pages and slots of requests that ended are used again."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    root = Path(__file__).resolve().parent.parent
+    folder = models.make_folder(tmp_path / "m", models.CONFIGS["A"], seed=6)
+    cfg, weights = models.read_folder(folder)
+    requests = {"x": random_tokens(50, cfg["vocab"], 1), "y": random_tokens(90, cfg["vocab"], 2), "z": random_tokens(20, cfg["vocab"], 3),
+                "u": random_tokens(70, cfg["vocab"], 4), "v": random_tokens(33, cfg["vocab"], 5)}
+    truth, scale = truth_of(cfg, weights, requests)
+    tol = FP32_TOL if dtype == "float32" else bfloat16_bounds(cfg, weights, requests, truth, scale)[0]
+    steps = schedules.mixed(requests, max_live=2)
+    out = tmp_path / "out"
+    proc = subprocess.run(
+        [sys.executable, str(root / "bin" / "trace_run"), "--model", str(folder), "--dtype", dtype, "--out", str(out),
+         "--max-tokens", str(schedules.max_live_tokens(steps))],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done ")] == [f"done {i}" for i in range(len(steps))]
+    for step, rows in zip(steps, schedules.positions_of(steps)):
+        if not rows:  # (a step in which nothing is wanted writes no file)
+            assert not (out / f"{step['step']}.f32").exists()
+            continue
+        got = torch.from_numpy(np.fromfile(out / f"{step['step']}.f32", dtype="<f4").reshape(len(rows), -1))
+        for row, (rid, pos) in zip(got, rows):
+            assert distance(row, truth[rid][pos], scale) < tol
+
+
 def drawn_config(seed: int) -> dict:
     """A configuration drawn from a seed: the order of layers, every size and constant."""
     rng = random.Random(seed)

@@ -46,11 +46,14 @@ struct PrepArgs {
   int page_size;
 };
 
-// kPrepChan: channels a lane holds (the widest head of the launch over 64, rounded up to a power of two).
-template <typename T, int kPrepChan>
-__global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const PrepArgs<T> a) {
+// kPrepChan: channels a lane holds (the widest head of the launch over 64, rounded up to a power of two).  kPrepTok:
+// consecutive tokens a wave takes for its head, all their loads asked for before anything is computed: a wave has
+// a few hundred bytes of one (token, head) to fetch, and with one token a wave the bytes in flight on the whole GPU
+// are what bounds the kernel.
+template <typename T, int kPrepChan, int kPrepTok>
+__global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const PrepArgs<T> a, int n_tokens) {
   __shared__ float turned[kPrepWaves][kPrepChan * kWave];
-  const int t = blockIdx.x;
+  const int t0 = blockIdx.x * kPrepTok;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int unit = blockIdx.y * kPrepWaves + wave;
   const int n_units = a.n_q + a.n_kv + (a.dv > 0 ? a.n_kv : 0);
@@ -58,125 +61,136 @@ __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const P
   const bool is_q = live && unit < a.n_q;
   const bool is_k = live && !is_q && unit < a.n_q + a.n_kv;
   const bool is_v = live && !is_q && !is_k;
-  T* base = a.rows + (size_t)t * a.row_stride;
-  const int slot = a.slot_mapping ? a.slot_mapping[t] : -1;
-  const bool store = a.k_pages != nullptr && slot >= 0;
-  const size_t page = store ? slot / a.page_size : 0;
-  const int off = store ? slot % a.page_size : 0;
   const int width = is_v ? a.dv : a.dk;
-  T* head = is_v ? base + (size_t)(a.n_q + a.n_kv) * a.dk + (size_t)(unit - a.n_q - a.n_kv) * a.dv
-                 : base + (size_t)(live ? unit : 0) * a.dk;
+  const int g = unit - a.n_q - a.n_kv;  // the kv head of a value unit
+  // where the unit's head starts in a row (an idle wave shadows the first head and stores nothing)
+  const size_t head_at = is_v ? (size_t)(a.n_q + a.n_kv) * a.dk + (size_t)g * a.dv : (size_t)(live ? unit : 0) * a.dk;
+  const float* w = is_q ? a.q_w : (is_k ? a.k_w : nullptr);
+  const bool mixes = is_v && a.v_first != nullptr;
   // every load is made whatever the head's width (a channel past the end is the head's first once more, and not
   // used), and nothing looks at a loaded value before all are asked for: a select right behind a load makes the
   // wave wait for each load in turn
-  const float* w = is_q ? a.q_w : (is_k ? a.k_w : nullptr);
-  const T* head_bias = a.bias ? a.bias + (head - base) : nullptr;
-  T raw[kPrepChan], raw_bias[kPrepChan];
+  T raw[kPrepTok][kPrepChan], first[kPrepTok][kPrepChan], raw_bias[kPrepChan];
   float wv[kPrepChan];
+  int slot[kPrepTok], pos[kPrepTok];
 #pragma unroll
-  for (int c = 0; c < kPrepChan; ++c) {
-    const int d = lane + c * kWave;
-    raw[c] = head[d < width ? d : 0];
-    if (head_bias) raw_bias[c] = head_bias[d < width ? d : 0];  // (uniform)
-    if (w) wv[c] = w[d < a.norm_dims ? d : 0];                  // (uniform)
-  }
-  float val[kPrepChan];
-  float ss = 0.f;
-#pragma unroll
-  for (int c = 0; c < kPrepChan; ++c) {
-    const int d = lane + c * kWave;
-    val[c] = (live && d < width) ? to_f32(raw[c]) : 0.f;
-    // (the sum is rounded to the rows' type, as a projection with a bias would have stored it)
-    if (head_bias && live && d < width) val[c] = to_f32(from_f32<T>(val[c] + to_f32(raw_bias[c])));
-    if (d < a.norm_dims) ss += val[c] * val[c];
-  }
-  if (w != nullptr) {  // (uniform per wave)
-    ss = wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / (float)a.norm_dims + a.eps);
+  for (int j = 0; j < kPrepTok; ++j) {
+    const int t = t0 + j < n_tokens ? t0 + j : n_tokens - 1;  // (tokens past the end: the last once more, not stored)
+    const T* head = a.rows + (size_t)t * a.row_stride + head_at;
+    slot[j] = a.slot_mapping ? a.slot_mapping[t] : -1;
+    pos[j] = a.temp_coef != 0.f ? a.positions[t] : 0;
 #pragma unroll
     for (int c = 0; c < kPrepChan; ++c) {
       const int d = lane + c * kWave;
-      if (d < a.norm_dims) val[c] = val[c] * inv * wv[c];
+      raw[j][c] = head[d < width ? d : 0];
+      if (mixes) first[j][c] = a.v_first[(size_t)t * a.v_first_stride + (size_t)g * a.dv + (d < width ? d : 0)];  // (uniform)
     }
   }
-  // rotation: every lane needs its partner's channel as it is after the norm
-  const bool turns = (is_q || is_k) && a.rot > 0;
-  if (a.rot > 0) {  // (uniform over the block)
 #pragma unroll
-    for (int c = 0; c < kPrepChan; ++c) turned[wave][lane + c * kWave] = val[c];
-    __syncthreads();
+  for (int c = 0; c < kPrepChan; ++c) {
+    const int d = lane + c * kWave;
+    if (a.bias) raw_bias[c] = a.bias[head_at + (d < width ? d : 0)];  // (uniform)
+    if (w) wv[c] = w[d < a.norm_dims ? d : 0];                        // (uniform)
   }
-  if (turns) {
-    const int rh = a.rot / 2;
+#pragma unroll
+  for (int j = 0; j < kPrepTok; ++j) {
+    const int t = t0 + j;
+    const bool there = live && t < n_tokens;
+    T* head = a.rows + (size_t)(t < n_tokens ? t : n_tokens - 1) * a.row_stride + head_at;
+    float val[kPrepChan];
+    float ss = 0.f;
 #pragma unroll
     for (int c = 0; c < kPrepChan; ++c) {
       const int d = lane + c * kWave;
-      const int r = d - a.rot_off;
-      if (d < width && r >= 0 && r < a.rot) {
-        int i, partner;
-        bool first;
-        if (a.pairing == 0) {
-          i = r / 2; first = (r % 2) == 0; partner = first ? d + 1 : d - 1;
-        } else {
-          first = r < rh; i = first ? r : r - rh; partner = first ? d + rh : d - rh;
+      val[c] = (live && d < width) ? to_f32(raw[j][c]) : 0.f;
+      // (the sum is rounded to the rows' type, as a projection with a bias would have stored it)
+      if (a.bias && live && d < width) val[c] = to_f32(from_f32<T>(val[c] + to_f32(raw_bias[c])));
+      if (d < a.norm_dims) ss += val[c] * val[c];
+    }
+    if (w != nullptr) {  // (uniform per wave)
+      ss = wave_sum(ss);
+      const float inv = 1.0f / sqrtf(ss / (float)a.norm_dims + a.eps);
+#pragma unroll
+      for (int c = 0; c < kPrepChan; ++c) {
+        const int d = lane + c * kWave;
+        if (d < a.norm_dims) val[c] = val[c] * inv * wv[c];
+      }
+    }
+    // rotation: every lane needs its partner's channel as it is after the norm
+    if (a.rot > 0) {  // (uniform over the block)
+      if (j > 0) __syncthreads();  // everybody has read the token before
+#pragma unroll
+      for (int c = 0; c < kPrepChan; ++c) turned[wave][lane + c * kWave] = val[c];
+      __syncthreads();
+      if (is_q || is_k) {
+        const int rh = a.rot / 2;
+        const size_t row = (size_t)(t < n_tokens ? t : n_tokens - 1) * rh;
+#pragma unroll
+        for (int c = 0; c < kPrepChan; ++c) {
+          const int d = lane + c * kWave;
+          const int r = d - a.rot_off;
+          if (d < width && r >= 0 && r < a.rot) {
+            int i, partner;
+            bool one;
+            if (a.pairing == 0) {
+              i = r / 2; one = (r % 2) == 0; partner = one ? d + 1 : d - 1;
+            } else {
+              one = r < rh; i = one ? r : r - rh; partner = one ? d + rh : d - rh;
+            }
+            const float o = turned[wave][partner];
+            const float2 cs = a.cos_sin[row + i];
+            val[c] = one ? val[c] * cs.x - o * cs.y : val[c] * cs.x + o * cs.y;
+          }
         }
-        const float o = turned[wave][partner];
-        const float2 cs = a.cos_sin[(size_t)t * rh + i];
-        val[c] = first ? val[c] * cs.x - o * cs.y : val[c] * cs.x + o * cs.y;
       }
     }
-  }
-  if (!live) return;
-  if (is_q) {
-    float f = 1.0f;
-    if (a.temp_coef != 0.f) f = 1.0f + a.temp_coef * logf((float)((a.positions[t] + 1) / a.temp_every + 1));
+    if (!there) continue;
+    const bool store = a.k_pages != nullptr && slot[j] >= 0;
+    const size_t page = store ? slot[j] / a.page_size : 0;
+    const int off = store ? slot[j] % a.page_size : 0;
+    if (is_q) {
+      float f = 1.0f;
+      if (a.temp_coef != 0.f) f = 1.0f + a.temp_coef * logf((float)((pos[j] + 1) / a.temp_every + 1));
 #pragma unroll
-    for (int c = 0; c < kPrepChan; ++c) {
-      const int d = lane + c * kWave;
-      if (d < width) head[d] = from_f32<T>(val[c] * f);
+      for (int c = 0; c < kPrepChan; ++c) {
+        const int d = lane + c * kWave;
+        if (d < width) head[d] = from_f32<T>(val[c] * f);
+      }
+      continue;
     }
-    return;
-  }
-  if (is_k) {
-    if (a.k_pages != nullptr && !store) return;  // a token without a slot keeps nothing
-    T* dst = store ? a.k_pages + ((page * a.n_kv + (unit - a.n_q)) * a.page_size + off) * a.dk : head;
+    if (is_k) {
+      if (a.k_pages != nullptr && !store) continue;  // a token without a slot keeps nothing
+      T* dst = store ? a.k_pages + ((page * a.n_kv + (unit - a.n_q)) * a.page_size + off) * a.dk : head;
 #pragma unroll
-    for (int c = 0; c < kPrepChan; ++c) {
-      const int d = lane + c * kWave;
-      if (d < width) dst[d] = from_f32<T>(val[c]);
+      for (int c = 0; c < kPrepChan; ++c) {
+        const int d = lane + c * kWave;
+        if (d < width) dst[d] = from_f32<T>(val[c]);
+      }
+      continue;
     }
-    return;
-  }
-  // a value head
-  const int g = unit - a.n_q - a.n_kv;
-  if (a.v_first == nullptr && a.bias != nullptr) {  // (values with a bias and no mixing go back too: later layers may read them)
+    // a value head
+    if (mixes) {
+      const float lam = a.lam[0];
 #pragma unroll
-    for (int c = 0; c < kPrepChan; ++c) {
-      const int d = lane + c * kWave;
-      if (d < width) head[d] = from_f32<T>(val[c]);
-    }
-  }
-  if (a.v_first != nullptr) {
-    const float lam = a.lam[0];
-    const T* vf = a.v_first + (size_t)t * a.v_first_stride + (size_t)g * a.dv;
-    T first[kPrepChan];
-#pragma unroll
-    for (int c = 0; c < kPrepChan; ++c) first[c] = vf[lane + c * kWave < width ? lane + c * kWave : 0];
-#pragma unroll
-    for (int c = 0; c < kPrepChan; ++c) {
-      const int d = lane + c * kWave;
-      if (d < width) {
-        val[c] = (1.0f - lam) * val[c] + lam * to_f32(first[c]);
-        head[d] = from_f32<T>(val[c]);
+      for (int c = 0; c < kPrepChan; ++c) {
+        const int d = lane + c * kWave;
+        if (d < width) val[c] = (1.0f - lam) * val[c] + lam * to_f32(first[j][c]);
       }
     }
-  }
-  if (store && a.v_pages != nullptr) {
-    T* dst = a.v_pages + ((page * a.n_kv + g) * a.page_size + off) * a.dv;
+    if (mixes || a.bias != nullptr) {  // (what changed goes back: later layers may read these values)
 #pragma unroll
-    for (int c = 0; c < kPrepChan; ++c) {
-      const int d = lane + c * kWave;
-      if (d < width) dst[d] = from_f32<T>(val[c]);
+      for (int c = 0; c < kPrepChan; ++c) {
+        const int d = lane + c * kWave;
+        if (d < width) head[d] = from_f32<T>(val[c]);
+      }
+    }
+    if (store && a.v_pages != nullptr) {
+      T* dst = a.v_pages + ((page * a.n_kv + g) * a.page_size + off) * a.dv;
+#pragma unroll
+      for (int c = 0; c < kPrepChan; ++c) {
+        const int d = lane + c * kWave;
+        if (d < width) dst[d] = from_f32<T>(val[c]);
+      }
     }
   }
 }
@@ -399,22 +413,27 @@ TL_EXPORT int tl_head_prepare(void* rows, int row_stride, int n_tokens, int n_q,
   TL_REQUIRE(k_pages == nullptr || (slot_mapping != nullptr && page_size > 0 && (dv == 0 || v_pages != nullptr)), "head_prepare: pages without slots");
   if (n_tokens == 0) return TL_OK;
   const int units = n_q + n_kv + (dv > 0 ? n_kv : 0);
-  const dim3 grid(n_tokens, (units + kPrepWaves - 1) / kPrepWaves);
   const int widest = dk > dv ? dk : dv;
+  // four tokens a wave while a lane holds few channels and the launch still has blocks for every CU several times over
+  const bool four = widest <= 4 * kWave && (long long)n_tokens * units >= 64LL * tl_device_facts().compute_units;
+  const int tok = four ? 4 : 1;
+  const dim3 grid((n_tokens + tok - 1) / tok, (units + kPrepWaves - 1) / kPrepWaves);
+#define TL_PREP_LAUNCH(T, CH, TOK) head_prepare_kernel<T, CH, TOK><<<grid, kPrepWaves * kWave, 0, stream>>>(a, n_tokens)
 #define TL_PREP(T)                                                                                                   \
   do {                                                                                                               \
-    PrepArgs<T> a{(T*)rows, row_stride, n_q, n_kv, dk, dv, (const T*)bias, q_w, k_w, (q_w || k_w) ? norm_dims : 0, eps,              \
+    PrepArgs<T> a{(T*)rows, row_stride, n_q, n_kv, dk, dv, (const T*)bias, q_w, k_w, (q_w || k_w) ? norm_dims : 0, eps, \
                   (const float2*)cos_sin, rot_off, rot, pairing, positions, temp_coef, temp_every, (const T*)v_first, \
                   v_first_stride, lam, (T*)k_pages, (T*)v_pages, slot_mapping, page_size};                           \
-    if (widest <= kWave) head_prepare_kernel<T, 1><<<grid, kPrepWaves * kWave, 0, stream>>>(a);                      \
-    else if (widest <= 2 * kWave) head_prepare_kernel<T, 2><<<grid, kPrepWaves * kWave, 0, stream>>>(a);             \
-    else if (widest <= 4 * kWave) head_prepare_kernel<T, 4><<<grid, kPrepWaves * kWave, 0, stream>>>(a);             \
-    else if (widest <= 8 * kWave) head_prepare_kernel<T, 8><<<grid, kPrepWaves * kWave, 0, stream>>>(a);             \
-    else head_prepare_kernel<T, kPrepMaxChan><<<grid, kPrepWaves * kWave, 0, stream>>>(a);                           \
+    if (widest <= kWave) { if (four) TL_PREP_LAUNCH(T, 1, 4); else TL_PREP_LAUNCH(T, 1, 1); }                        \
+    else if (widest <= 2 * kWave) { if (four) TL_PREP_LAUNCH(T, 2, 4); else TL_PREP_LAUNCH(T, 2, 1); }               \
+    else if (widest <= 4 * kWave) { if (four) TL_PREP_LAUNCH(T, 4, 4); else TL_PREP_LAUNCH(T, 4, 1); }               \
+    else if (widest <= 8 * kWave) TL_PREP_LAUNCH(T, 8, 1);                                                           \
+    else TL_PREP_LAUNCH(T, kPrepMaxChan, 1);                                                                         \
   } while (0)
   if (dtype == TL_F32) TL_PREP(float);
   else if (dtype == TL_BF16) TL_PREP(bf16_t);
   else return tl_fail(TL_ERR_ARG, "head_prepare: unknown dtype %d", dtype);
+#undef TL_PREP_LAUNCH
 #undef TL_PREP
   return tl_check_launch("head_prepare");
 }
