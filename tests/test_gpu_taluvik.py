@@ -18,7 +18,7 @@ from .test_gpu_engine import run_trace
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [70, 41, 100, 35, 50, 33], "B": [66, 40, 130, 35, 90], "C": [45, 150, 37, 64, 120]}
-#: distances are measured as the checker of a replay would: the difference of two rows of logits with
+#: distances are measured as a replay of a trace is judged: the difference of two rows of logits with
 #: its mean taken off, root mean square over the vocabulary, over the root mean square of the truth
 FP32_TOL = 2e-5
 BF16_TOL = 4e-2

@@ -19,7 +19,7 @@ from .test_gpu_engine import run_trace
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [70, 41, 100, 35, 50, 33], "B": [66, 40, 130, 35, 90], "C": [45, 150, 37, 64, 120]}
-#: distances are measured as a replay's checker would: the difference of two rows of logits with its mean
+#: distances are measured as a replay of a trace is judged: the difference of two rows of logits with its mean
 #: taken off, root mean square over the vocabulary, over the root mean square of the truth
 FP32_TOL = 2e-5
 BF16_TOL = 4e-2
@@ -291,6 +291,10 @@ def test_branch_norm_and_the_other_small_kernels(dtype):
     rows = ops.branch_norm_add(d_stream, y.to(dev), w.to(dev), 1e-5)
     torch.testing.assert_close(d_stream.cpu().double(), want, rtol=1e-6, atol=1e-6)
     assert rows.dtype == dtype and torch.equal(rows.cpu(), d_stream.cpu().to(dtype))
+    # a launch of many rows takes another form of the kernel than one of few: the same bits row by row
+    many_stream, many_y = stream.repeat(20, 1).to(dev), y.repeat(20, 1).to(dev)
+    ops.branch_norm_add(many_stream, many_y, w.to(dev), 1e-5)
+    assert many_stream.shape[0] > 512 and torch.equal(many_stream[:n].cpu(), d_stream.cpu()) and torch.equal(many_stream[-n:].cpu(), d_stream.cpu())
     # a norm of some columns of a wider matrix, of gathered rows of a 32-bit matrix
     wide = torch.randn((n, hidden + 40), generator=g)
     idx = torch.tensor([5, 0, 36, 5], dtype=torch.int32)
@@ -374,6 +378,26 @@ def test_one_far_key_stands_out_when_values_lie_inside_the_keys(form, dtype):
                 if special[i] <= p:
                     assert float(w[special[i]]) > 0.99  # the inputs do single that key out
                     torch.testing.assert_close(out[t, h], k_all[special[i], off : off + dv], rtol=0.05, atol=0.05)
+
+
+def test_float32_bits_do_not_depend_on_the_rows_of_a_step(tmp_path):
+    """A prompt of more rows than the kernels' forms for few rows take, whole, against the same tokens in a long
+    portion, a short one and single tokens: kernels that have a form for few rows and one for many add alike."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    folder = models.make_folder(tmp_path / "m", models.CONFIGS["A"], seed=2)
+    cfg, _ = models.read_folder(folder)
+    tokens = random_tokens(660, cfg["vocab"], 4)
+    engine = Engine.from_folder(folder, dtype="float32", page_size=16, num_pages=96, max_seqs=2)
+    engine.admit("whole")
+    whole = engine.step([StepEntry("whole", tokens, list(range(len(tokens))))]).cpu()
+    engine.admit("cut")
+    rows, at = [], 0
+    for n in [560, 70] + [1] * 30:
+        rows.append(engine.step([StepEntry("cut", tokens[at : at + n], list(range(n)))]).cpu())
+        at += n
+    assert at == len(tokens)
+    assert torch.equal(torch.cat(rows), whole)
 
 
 # ----------------------------------------------------------------------------- long decoding, generation, drawn configurations

@@ -52,6 +52,7 @@ struct PrepArgs {
 // are what bounds the kernel.
 template <typename T, int kPrepChan, int kPrepTok>
 __global__ void __launch_bounds__(kPrepWaves* kWave) head_prepare_kernel(const PrepArgs<T> a, int n_tokens) {
+#pragma clang fp contract(off)  // the same operations in every instantiation: a head's result does not depend on the launch's form
   __shared__ float turned[kPrepWaves][kPrepChan * kWave];
   const int t0 = blockIdx.x * kPrepTok;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
@@ -208,6 +209,7 @@ template <typename T, int kRowHeld>
 __global__ void __launch_bounds__(kRowThreads)
 branch_norm_add_held_kernel(float* __restrict__ stream, const T* __restrict__ y, const float* __restrict__ w,
                             T* __restrict__ rows, int hidden, float eps) {
+#pragma clang fp contract(off)  // operation for operation the kernel below: no multiply-add is fused in one and not the other
   __shared__ float scratch[kRowThreads / kWave];
   const size_t r = blockIdx.x;
   const T* yr = y + r * hidden;
@@ -248,6 +250,7 @@ template <typename T>
 __global__ void __launch_bounds__(kRowThreads)
 branch_norm_add_kernel(float* __restrict__ stream, const T* __restrict__ y, const float* __restrict__ w,
                        T* __restrict__ rows, int hidden, float eps) {
+#pragma clang fp contract(off)
   __shared__ float scratch[kRowThreads / kWave];
   const size_t r = blockIdx.x;
   const T* yr = y + r * hidden;
@@ -272,6 +275,7 @@ template <typename XT, typename T>
 __global__ void __launch_bounds__(kRowThreads)
 rmsnorm_columns_kernel(const XT* __restrict__ x, int x_stride, const int32_t* __restrict__ rows,
                        const float* __restrict__ w, T* __restrict__ y, int y_stride, int width, float eps) {
+#pragma clang fp contract(off)
   __shared__ float scratch[kRowThreads / kWave];
   const size_t r = blockIdx.x;
   const size_t s = rows ? (size_t)rows[r] : r;
