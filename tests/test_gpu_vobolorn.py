@@ -457,6 +457,56 @@ def test_greedy_generation_through_the_entry_point(tmp_path):
         assert logits[r.token_ids[0]] >= logits.max() - 0.05 * float(logits.std())
 
 
+def test_a_preempted_request_is_computed_again_with_the_same_tokens(tmp_path):
+    """Too few pages for four requests: the scheduler takes the youngest off, gives its pages and its slot away and
+    later computes it again from its prompt and what it had generated (keys, latent rows and mixed values land in
+    other pages): the sampled tokens are those of the run with room for everybody."""
+    from torchllms_amd.inference import LLM
+
+    folder = models.make_folder(tmp_path / "m", models.CONFIGS["A"], seed=9)
+    cfg, _ = models.read_folder(folder)
+    prompts = [random_tokens(n, cfg["vocab"], 80 + n) for n in (30, 25, 28, 21)]
+    ample = LLM(str(folder), precision="float32", max_len=96, max_bsz=4, page_size=8)
+    want = ample.generate(prompt_token_ids=prompts, temperature=0.8, max_new_tokens=30, seed=7)
+    tight = LLM(str(folder), precision="float32", max_len=96, max_bsz=4, page_size=8, num_pages=20)  # 160 places for 224 tokens
+    got = tight.generate(prompt_token_ids=prompts, temperature=0.8, max_new_tokens=30, seed=7)
+    assert tight.last_stats["preemptions"] > 0
+    assert [r.token_ids for r in got] == [r.token_ids for r in want]
+    tight.engine.cache.check_invariants()
+
+
+def test_generate_command_line_with_random_weights(tmp_path):
+    """The generate program given nothing but a config.json: ``--random-weights --seed`` draws the weights that
+    ``write_model_folder`` would write for that seed, so the plain model can say which tokens to expect."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from torchllms_amd.config.vobolorn import VobolornConfig
+    from torchllms_amd.weights import write_model_folder
+
+    root = Path(__file__).resolve().parent.parent
+    folder = tmp_path / "only_config"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(models.CONFIGS["B"]))
+    prompt = random_tokens(13, models.CONFIGS["B"]["vocab"], 21)
+    proc = subprocess.run(
+        [sys.executable, "-m", "torchllms_amd.inference.generate", "--model", str(folder), "--dtype", "float32", "--random-weights",
+         "--seed", "7", "--max-new-tokens", "6", "--prompt-ids", *map(str, prompt)],
+        capture_output=True, text=True, cwd=root, timeout=300,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [int(t) for t in proc.stdout.split()[-6:]]
+    written = write_model_folder(tmp_path / "written", VobolornConfig.from_dict(models.CONFIGS["B"]), seed=7, dtype=torch.float32)
+    cfg, weights = models.read_folder(written)
+    w64 = {k: v.double() for k, v in weights.items()}
+    toks = list(prompt)
+    for _ in range(6):
+        toks.append(int(plain.forward(cfg, w64, toks)[-1].argmax()))
+    assert got == toks[len(prompt):]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_replay_program(tmp_path, dtype):
     """``bin/trace_run`` as a process: steps in, logits files out, the plain model's values; the pool is made for
