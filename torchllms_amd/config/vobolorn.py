@@ -119,7 +119,11 @@ class VobolornConfig:
                 if not isinstance(qt, dict) or "coef" not in qt or "every" not in qt:
                     raise ConfigError(f"{where}: q_temp needs 'coef' and 'every'")
                 _number(where, "q_temp.coef", qt["coef"])
-                _positive_int(where, "q_temp.every", qt["every"])
+                every = qt["every"]
+                if isinstance(every, float) and every.is_integer():  # (64.0 is 64)
+                    every = int(every)
+                    mixer = dict(mixer, q_temp=dict(qt, every=every))
+                _positive_int(where, "q_temp.every", every)
         else:
             rot = mixer["rot"]
             if not isinstance(rot, dict) or "dims" not in rot or "base" not in rot:
